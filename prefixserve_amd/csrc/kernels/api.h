@@ -56,7 +56,7 @@ int psamd_rope_norm_kv_append(void* stream, void* qkv, int act_dtype, int64_t to
 int psamd_qk_prepare_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
                                const int32_t* positions, const float* table, int norm_dim, float eps, const float* bias,
                                const float* q_weight, const float* k_weight, int v_from_k, void* kv,
-                               const int32_t* write_slot);
+                               const int32_t* write_slot, int q_weight_per_head);
 
 // residual[r] += delta[r]; delta as for psamd_add_rmsnorm (one tensor in delta_dtype, or n_partials float32 slices).
 int psamd_residual_add(void* stream, float* residual, const void* delta, int delta_dtype, int n_partials,
@@ -108,19 +108,21 @@ int psamd_gated_scan(void* stream, const float* gates, const float* gate_b, cons
 
 // Mixture of experts. Router: z = x w_router^T in float (x in x_dtype, w_router float [E, K]), score =
 // sigmoid(z); chosen[t, :] = the top largest scores' experts (lower index among equals, largest
-// first), weight[t, :] = those scores.
+// first), weight[t, :] = those scores. bias (float [experts] or NULL) is added to z first. mode 1: the
+// choice is by z itself and the weights are the softmax over the chosen z alone.
 int psamd_moe_route(void* stream, const void* x, int x_dtype, const float* w_router, int32_t* chosen, float* weight,
-                    int64_t tokens, int K, int experts, int top);
+                    int64_t tokens, int K, int experts, int top, const float* bias, int mode);
 // The same choice from logits that a product has written (float [tokens, experts]).
 int psamd_moe_topk(void* stream, const float* logits, int32_t* chosen, float* weight, int64_t tokens, int experts,
-                   int top);
+                   int top, const float* bias, int mode);
 // Experts, one (token, choice) pair at a time: h = weight[t, j] * x[t]; g = min(gate h, limit), u =
 // clamp(up h, -limit, limit); act[t * top + j] = g * sigmoid(gate_alpha * g) * (u + up_shift);
 // out[j][t] = down act (float). w_gate_up is [E, 2F, K] (gate rows, then up rows), w_down [E, K, F].
+// weight_on_output: h = x[t] and out[j][t] = weight[t, j] * down act instead.
 int psamd_moe_experts_rows(void* stream, const void* x, const int32_t* chosen, const float* weight,
                            const void* w_gate_up, const void* w_down, void* act, float* out, int dtype,
                            int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
-                           float up_shift);
+                           float up_shift, int weight_on_output);
 
 // The same for bfloat16 with the pairs sorted by expert and every expert's pairs run through its
 // matrices in tiles on the matrix cores. ints: scratch of pairs + 3 * psamd_moe_grouped_max_tiles(pairs,
@@ -130,11 +132,56 @@ int psamd_moe_grouped_max_tiles(int64_t pairs, int experts);
 int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen, const float* weight,
                               const void* w_gate_up, const void* w_down, void* act, float* out, int32_t* ints,
                               int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
-                              float up_shift, int grouped_already);
+                              float up_shift, int grouped_already, int weight_on_output);
 // psamd_moe_topk and the sorting of the pairs into `ints` in one workgroup, for up to 64 tokens;
 // psamd_moe_experts_grouped is then called with grouped_already = 1 and the same `ints`.
 int psamd_moe_topk_group(void* stream, const float* logits, int32_t* chosen, float* weight, int32_t* ints, int64_t tokens,
-                         int experts, int top);
+                         int experts, int top, const float* bias, int mode);
+// out[t, :] *= sigmoid(x[t] . w) for float out [tokens, out_hidden], x [tokens, hidden] in act_dtype, w float [hidden].
+int psamd_row_gate(void* stream, float* out, const void* x, int act_dtype, const float* w, int64_t tokens, int out_hidden,
+                   int hidden);
+
+// Layer norm with weight and bias (float [hidden] each) around the float32 residual stream:
+// if delta: residual[r] += LN_post(delta[r]) (delta as for psamd_add_rmsnorm); if out: out[r] = LN_pre(residual[r])
+// in out_dtype. rows (NULL or int32 [n_rows], without a delta): out[i] = LN_pre(residual[rows[i]]).
+int psamd_layernorm_step(void* stream, float* residual, const int32_t* rows, const void* delta, int delta_dtype,
+                         int n_partials, int64_t partial_stride, const float* post_w, const float* post_b, float post_eps,
+                         const float* pre_w, const float* pre_b, float pre_eps, void* out, int out_dtype, int64_t n_rows,
+                         int hidden);
+// x[t, e] += sin (e even) / cos (e odd) of positions[t] * freq[e / 2]; x float [tokens, hidden], freq double [(hidden + 1) / 2].
+int psamd_add_sinusoid(void* stream, float* x, const int32_t* positions, const double* freq, int64_t tokens, int hidden);
+
+// Short causal convolution per channel over each item's tokens: out[t, c] = act(sum_j taps_w[c, j] in[t - (taps - 1) + j, c]),
+// continued in front of an item's first token from the inputs its state slot saved (state[slot, j * channels + c],
+// oldest first), which are replaced by the item's last taps - 1 inputs. act 1 = SiLU, 0 = none. out is float.
+int psamd_short_conv(void* stream, const void* in, int act_dtype, int64_t in_row, const float* taps_w, float* out,
+                     int64_t out_row, float* state, int64_t state_row, const int32_t* tok_item, const int32_t* item_start,
+                     const int32_t* slots, int64_t tokens, int items, int channels, int taps, int act);
+// Operands of the gated delta rule: u row [q: groups x dim | k: groups x dim | ...] float, q and k made unit
+// vectors in place (q times q_scale); gates row [strength logits | decay inputs] (heads each) -> coef row
+// [g | -b | b]: b = sigmoid(.), g = exp(-exp(a_log[h]) softplus(. + dt_bias[h])).
+int psamd_gated_delta_prepare(void* stream, float* u, int64_t u_row, int groups, int dim, const float* gates,
+                              const float* a_log, const float* dt_bias, float* coef, int64_t tokens, int heads,
+                              float q_scale, float unit_eps);
+// Operands of the generalized delta rule from rows in act_dtype (r, k, v, removal logits: heads x dim at their
+// columns; the decay's low-rank inner values: rank at l_col) -> ops row [r | k | v | w | p | c] float.
+int psamd_general_delta_prepare(void* stream, const void* rows, int act_dtype, int64_t in_row, int r_col, int k_col,
+                                int v_col, int a_col, int l_col, const float* a_bias, const float* w2, const float* w0,
+                                float* ops, int64_t tokens, int heads, int dim, int rank, float decay_floor, float unit_eps);
+// The delta-rule recurrence over each item's tokens from its state slot (state[slot, (h * vdim + j) * dim + i]):
+// S' = d S; S = S' + (ps p)(c^T S*) + k (xs x)^T, S* = S' if reads_decayed else S; out = S^T r. k, c, p, r: float
+// vectors of `dim` per (token, key group), rows key_row apart; dvec (or NULL) per (token, head), dscal / pscal /
+// xscal (or NULL = 1) per (token, head), rows scal_row apart; x [.., heads x vdim] rows x_row apart; out likewise.
+int psamd_delta_scan(void* stream, const float* kvec, const float* cvec, const float* pvec, const float* rvec, int64_t key_row,
+                     int key_groups, const float* dvec, int64_t dvec_row, const float* dscal, const float* pscal,
+                     const float* xscal, int64_t scal_row, const float* x, int64_t x_row, float* out, int64_t out_row,
+                     float* state, int64_t state_row, const int32_t* item_start, const int32_t* slots, int items, int heads,
+                     int dim, int vdim, int reads_decayed);
+// out[t, h, :] = o[t, h, :] / sqrt(mean(o^2) + eps) * weight * act(gate[t, h, :]); o float, weight float [vdim]
+// (or [heads * vdim] with weight_per_head), gate rows gate_row apart in act_dtype, act 0 = SiLU, 1 = sigmoid.
+int psamd_heads_norm_gate(void* stream, const float* o, int64_t tokens, int heads, int vdim, const float* weight,
+                          int weight_per_head, float eps, const void* gate, int act_dtype, int64_t gate_row, int gate_act,
+                          void* out);
 
 // out[M, N] = x[M, K] * w[N, K]^T with float accumulation (LDS-tiled FMA; exact path and fallback).
 int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,

@@ -515,7 +515,7 @@ __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
     A* __restrict__ qkv, int hq, int hkv, int d, const int32_t* __restrict__ positions,
     const float2* __restrict__ table, int norm_dim, float eps, A* __restrict__ kv,
     const int32_t* __restrict__ write_slot, int group_lanes, const float* __restrict__ bias,
-    const float* __restrict__ q_weight, const float* __restrict__ k_weight, int v_from_k) {
+    const float* __restrict__ q_weight, const float* __restrict__ k_weight, int v_from_k, int q_weight_stride) {
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x & (kWave - 1);
   const int per_wave = kWave / group_lanes;
@@ -535,7 +535,8 @@ __global__ __launch_bounds__(256) void rope_norm_kv_append_kernel(
   const int64_t page_elems = 2LL * hkv * kPage * d;
   if (head < hq + hkv) {
     const int pos = positions[t];
-    const float* nw = head < hq ? q_weight : k_weight;
+    // q_weight_stride = d: every query head has a weight of its own (a number per head folded into it)
+    const float* nw = head < hq ? (q_weight != nullptr ? q_weight + static_cast<int64_t>(head) * q_weight_stride : nullptr) : k_weight;
     float a[2], b[2];
     float ss = 0.f;
 #pragma unroll
@@ -808,8 +809,9 @@ int psamd_to_activation(void* stream, const float* in, void* out, int act_dtype,
 int psamd_qk_prepare_kv_append(void* stream, void* qkv, int act_dtype, int64_t tokens, int hq, int hkv, int head_dim,
                                const int32_t* positions, const float* table, int norm_dim, float eps, const float* bias,
                                const float* q_weight, const float* k_weight, int v_from_k, void* kv,
-                               const int32_t* write_slot) {
+                               const int32_t* write_slot, int q_weight_per_head) {
   PSAMD_REQUIRE(tokens >= 0 && hq > 0 && hkv >= 0, "bad sizes");
+  const int q_weight_stride = q_weight_per_head ? head_dim : 0;
   PSAMD_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= 256, "head_dim must be even and at most 256");
   PSAMD_REQUIRE(norm_dim >= 0 && norm_dim <= head_dim, "norm_dim must be in [0, head_dim]");
   PSAMD_REQUIRE(kv == nullptr || (write_slot != nullptr && hkv > 0), "a cache needs write slots and kv heads");
@@ -826,11 +828,11 @@ int psamd_qk_prepare_kv_append(void* stream, void* qkv, int act_dtype, int64_t t
   if (act_dtype == kBF16) {
     rope_norm_kv_append_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(static_cast<bf16_t*>(qkv), hq, hkv, head_dim, positions,
                                                                  tab, norm_dim, eps, static_cast<bf16_t*>(kv), write_slot,
-                                                                 group_lanes, bias, q_weight, k_weight, v_from_k);
+                                                                 group_lanes, bias, q_weight, k_weight, v_from_k, q_weight_stride);
   } else if (act_dtype == kF32) {
     rope_norm_kv_append_kernel<float><<<grid, dim3(256), 0, s>>>(static_cast<float*>(qkv), hq, hkv, head_dim, positions,
                                                                 tab, norm_dim, eps, static_cast<float*>(kv), write_slot,
-                                                                group_lanes, bias, q_weight, k_weight, v_from_k);
+                                                                group_lanes, bias, q_weight, k_weight, v_from_k, q_weight_stride);
   } else {
     return fail("psamd_qk_prepare_kv_append: activation dtype must be float32 or bfloat16");
   }
@@ -841,7 +843,7 @@ int psamd_rope_norm_kv_append(void* stream, void* qkv, int act_dtype, int64_t to
                               const int32_t* positions, const float* table, int norm_dim, float eps, void* kv,
                               const int32_t* write_slot) {
   return psamd_qk_prepare_kv_append(stream, qkv, act_dtype, tokens, hq, hkv, head_dim, positions, table, norm_dim, eps,
-                                    nullptr, nullptr, nullptr, 0, kv, write_slot);
+                                    nullptr, nullptr, nullptr, 0, kv, write_slot, 0);
 }
 
 // residual[r] += delta[r] (delta as for psamd_add_rmsnorm: one tensor in delta_dtype or float32 slices).

@@ -8,10 +8,13 @@
 //   expert is read once per tile of pairs instead of once per pair: a decode batch reads each
 //   expert it uses once, a prompt's portion runs as grouped products.
 //
-// Router: score = sigmoid(x . w_r[e]) in float; the `top` largest are taken, the lower index
-// among equals. Expert: with h = weight * x, g = min(gate h, limit), u = clamp(up h, -limit, limit),
-// act = g * sigmoid(gate_alpha * g) * (u + up_shift), out = down act. The weight multiplies the
-// expert's input, so it cannot be pulled out of the clamps.
+// Router: z = x . w_r[e] (+ bias[e]) in float; the `top` largest are taken, the lower index among
+// equals. mode 0: the score is sigmoid(z) and is the weight as it is; mode 1: the weights are the
+// softmax over the chosen z alone. Expert: with h = weight * x, g = min(gate h, limit), u = clamp(up h,
+// -limit, limit), act = g * sigmoid(gate_alpha * g) * (u + up_shift), out = down act. There the weight
+// multiplies the expert's input, so it cannot be pulled out of the clamps; with weight_on_output the
+// expert sees x itself and the weight multiplies out (limit = infinity, gate_alpha = 1, up_shift = 0
+// then make the plain SiLU-gated expert).
 
 #include <algorithm>
 
@@ -63,28 +66,14 @@ __device__ __forceinline__ float wave_dot(const W* __restrict__ row, const float
 
 // ------------------------------------------------------------------ router
 
-// One block of four waves per token: the waves share the experts' dot products, then wave 0
-// picks the `top` largest scores one after the other (each pick: a strided scan and a wave
-// reduction that prefers the lower index among equals).
-template <typename A>
-__global__ __launch_bounds__(256) void moe_route_kernel(const A* __restrict__ x, const float* __restrict__ w_router,
-                                                        int32_t* __restrict__ chosen, float* __restrict__ weight,
-                                                        int K, int experts, int top) {
-  extern __shared__ __align__(16) float route_smem[];    // xs[K], score[experts]
-  float* xs = route_smem;
-  float* score = route_smem + K;
-  const int64_t t = blockIdx.x;
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
-  for (int i = threadIdx.x; i < K; i += blockDim.x) xs[i] = to_float<A>(x[t * K + i]);
-  __syncthreads();
-  for (int e = wave; e < experts; e += 4) {
-    const float z = wave_dot<float>(w_router + static_cast<int64_t>(e) * K, xs, K, lane);
-    if (lane == 0) score[e] = 1.f / (1.f + expf(-z));
-  }
-  __syncthreads();
-  if (wave != 0) return;
+// The router's choice for one token by one wave: score[] (LDS, `experts` entries: sigmoid(z) in mode
+// 0, z in mode 1) -> chosen / weight [top], largest first, the lower index among equals; taken
+// entries are overwritten. Mode 1 then turns the chosen z into their softmax.
+__device__ __forceinline__ void pick_top(float* score, int experts, int top, int mode, int32_t* __restrict__ chosen,
+                                         float* __restrict__ weight, int lane) {
+  const float kTaken = -__builtin_inff();
   for (int j = 0; j < top; ++j) {
-    float best = -1.f;                                   // scores lie in [0, 1]; taken ones are set to -2
+    float best = kTaken;
     int at = 0x7fffffff;
     for (int e = lane; e < experts; e += kWave) {
       const float s = score[e];
@@ -103,54 +92,63 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const A* __restrict__ x,
       }
     }
     if (lane == 0) {
-      chosen[t * top + j] = at;
-      weight[t * top + j] = best;
-      score[at] = -2.f;
+      chosen[j] = at;
+      weight[j] = best;
+      if (at != 0x7fffffff) score[at] = kTaken;
     }
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
   }
+  if (mode == 1 && lane == 0) {
+    const float m = weight[0];                           // the largest comes first
+    float sum = 0.f;
+    for (int j = 0; j < top; ++j) sum += expf(weight[j] - m);
+    for (int j = 0; j < top; ++j) weight[j] = expf(weight[j] - m) / sum;
+  }
 }
 
-// The same choice from logits a product has already written: z[t, :] float -> sigmoid, the `top`
-// largest. One wave per token, four tokens per block.
+__device__ __forceinline__ float router_score(float z, const float* __restrict__ bias, int e, int mode) {
+  if (bias != nullptr) z += bias[e];
+  return mode == 0 ? 1.f / (1.f + expf(-z)) : z;
+}
+
+// One block of four waves per token: the waves share the experts' dot products, then wave 0
+// picks the `top` largest scores one after the other (each pick: a strided scan and a wave
+// reduction that prefers the lower index among equals).
+template <typename A>
+__global__ __launch_bounds__(256) void moe_route_kernel(const A* __restrict__ x, const float* __restrict__ w_router,
+                                                        int32_t* __restrict__ chosen, float* __restrict__ weight,
+                                                        int K, int experts, int top, const float* __restrict__ bias, int mode) {
+  extern __shared__ __align__(16) float route_smem[];    // xs[K], score[experts]
+  float* xs = route_smem;
+  float* score = route_smem + K;
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < K; i += blockDim.x) xs[i] = to_float<A>(x[t * K + i]);
+  __syncthreads();
+  for (int e = wave; e < experts; e += 4) {
+    const float z = wave_dot<float>(w_router + static_cast<int64_t>(e) * K, xs, K, lane);
+    if (lane == 0) score[e] = router_score(z, bias, e, mode);
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  pick_top(score, experts, top, mode, chosen + t * top, weight + t * top, lane);
+}
+
+// The same choice from logits a product has already written (z[t, :] float). One wave per token,
+// four tokens per block.
 __global__ __launch_bounds__(256) void moe_topk_kernel(const float* __restrict__ z, int32_t* __restrict__ chosen,
-                                                       float* __restrict__ weight, int64_t tokens, int experts, int top) {
+                                                       float* __restrict__ weight, int64_t tokens, int experts, int top,
+                                                       const float* __restrict__ bias, int mode) {
   extern __shared__ __align__(16) float topk_smem[];     // score[4][experts]
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
   const int64_t t = static_cast<int64_t>(blockIdx.x) * 4 + wave;
   if (t >= tokens) return;
   float* score = topk_smem + wave * experts;
-  for (int e = lane; e < experts; e += kWave) score[e] = 1.f / (1.f + expf(-z[t * experts + e]));
+  for (int e = lane; e < experts; e += kWave) score[e] = router_score(z[t * experts + e], bias, e, mode);
   __builtin_amdgcn_wave_barrier();
   __threadfence_block();
-  for (int j = 0; j < top; ++j) {
-    float best = -1.f;
-    int at = 0x7fffffff;
-    for (int e = lane; e < experts; e += kWave) {
-      const float s = score[e];
-      if (s > best) {
-        best = s;
-        at = e;
-      }
-    }
-#pragma unroll
-    for (int o = kWave / 2; o > 0; o >>= 1) {
-      const float ob = __shfl_xor(best, o, kWave);
-      const int oa = __shfl_xor(at, o, kWave);
-      if (ob > best || (ob == best && oa < at)) {
-        best = ob;
-        at = oa;
-      }
-    }
-    if (lane == 0) {
-      chosen[t * top + j] = at;
-      weight[t * top + j] = best;
-      score[at] = -2.f;
-    }
-    __builtin_amdgcn_wave_barrier();
-    __threadfence_block();
-  }
+  pick_top(score, experts, top, mode, chosen + t * top, weight + t * top, lane);
 }
 
 // ------------------------------------------------------------------ experts, pair by pair
@@ -164,13 +162,13 @@ template <typename A>
 __global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(
     const A* __restrict__ x, const int32_t* __restrict__ chosen, const float* __restrict__ weight,
     const A* __restrict__ w_gate_up, A* __restrict__ act, int K, int F, int experts, int top, float gate_alpha,
-    float limit, float up_shift) {
+    float limit, float up_shift, int weight_on_output) {
   extern __shared__ __align__(16) float rows_smem[];     // h[K]
   const int64_t pair = blockIdx.x;
   const int64_t t = pair / top;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
   const int e = min(max(chosen[pair], 0), experts - 1);
-  const float wgt = weight[pair];
+  const float wgt = weight_on_output ? 1.f : weight[pair];
   for (int i = threadIdx.x; i < K; i += blockDim.x) rows_smem[i] = wgt * to_float<A>(x[t * K + i]);
   __syncthreads();
   const A* we = w_gate_up + static_cast<int64_t>(e) * 2 * F * K;
@@ -190,7 +188,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(
 template <typename A>
 __global__ __launch_bounds__(256) void moe_down_rows_kernel(
     const A* __restrict__ act, const int32_t* __restrict__ chosen, const A* __restrict__ w_down,
-    float* __restrict__ out, int64_t tokens, int K, int F, int experts, int top) {
+    float* __restrict__ out, int64_t tokens, int K, int F, int experts, int top, const float* __restrict__ out_weight) {
   extern __shared__ __align__(16) float rows_smem[];     // act[F]
   const int64_t pair = blockIdx.x;
   const int64_t t = pair / top;
@@ -206,7 +204,7 @@ __global__ __launch_bounds__(256) void moe_down_rows_kernel(
     const int k = static_cast<int>(blockIdx.y) * kRowsPerBlock + wave * kRowsPerWave + r;
     if (k >= K) break;
     const float v = wave_dot<A>(we + static_cast<int64_t>(k) * F, rows_smem, F, lane);
-    if (lane == 0) o[k] = v;
+    if (lane == 0) o[k] = out_weight != nullptr ? out_weight[pair] * v : v;
   }
 }
 
@@ -269,41 +267,16 @@ __global__ __launch_bounds__(1024) void moe_topk_group_kernel(const float* __res
                                                               float* __restrict__ weight, int tokens, int experts, int top,
                                                               int tile_rows, int max_tiles, int32_t* __restrict__ sorted,
                                                               int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_first,
-                                                              int32_t* __restrict__ tile_count) {
+                                                              int32_t* __restrict__ tile_count, const float* __restrict__ bias,
+                                                              int mode) {
   extern __shared__ int32_t group_smem[];      // as above, then score[16][experts]
   float* score = reinterpret_cast<float*>(group_smem + 4 * experts + 1) + (threadIdx.x >> 6) * experts;
   const int lane = threadIdx.x & (kWave - 1);
   for (int t = threadIdx.x >> 6; t < tokens; t += 16) {
-    for (int e = lane; e < experts; e += kWave) score[e] = 1.f / (1.f + expf(-z[static_cast<int64_t>(t) * experts + e]));
+    for (int e = lane; e < experts; e += kWave) score[e] = router_score(z[static_cast<int64_t>(t) * experts + e], bias, e, mode);
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
-    for (int j = 0; j < top; ++j) {
-      float best = -1.f;
-      int at = 0x7fffffff;
-      for (int e = lane; e < experts; e += kWave) {
-        const float s = score[e];
-        if (s > best) {
-          best = s;
-          at = e;
-        }
-      }
-#pragma unroll
-      for (int o = kWave / 2; o > 0; o >>= 1) {
-        const float ob = __shfl_xor(best, o, kWave);
-        const int oa = __shfl_xor(at, o, kWave);
-        if (ob > best || (ob == best && oa < at)) {
-          best = ob;
-          at = oa;
-        }
-      }
-      if (lane == 0) {
-        chosen[t * top + j] = at;
-        weight[t * top + j] = best;
-        score[at] = -2.f;
-      }
-      __builtin_amdgcn_wave_barrier();
-      __threadfence_block();
-    }
+    pick_top(score, experts, top, mode, chosen + t * top, weight + t * top, lane);
   }
   __threadfence_block();
   __syncthreads();                             // the workgroup's own writes of `chosen` are read below
@@ -444,7 +417,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
   for (int mt = 0; mt < MT; ++mt) {
     const int pair = pair_s[mt * 16 + r];
     if (pair < 0) continue;
-    const float pw = GATED ? pair_weight[pair] : 1.f;
+    const float pw = pair_weight != nullptr ? pair_weight[pair] : 1.f;   // on the input's sums (GATED) or on the output's
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const int nc = n0 + rt * 16 + 4 * g;
@@ -467,11 +440,11 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
       } else {
         float* o = out_f32 + (static_cast<int64_t>(pair % top) * tokens + pair / top) * N + nc;
         if (nc + 3 < N && (N & 3) == 0) {
-          *reinterpret_cast<float4*>(o) = float4{acc_g[rt][mt][0], acc_g[rt][mt][1], acc_g[rt][mt][2], acc_g[rt][mt][3]};
+          *reinterpret_cast<float4*>(o) = float4{pw * acc_g[rt][mt][0], pw * acc_g[rt][mt][1], pw * acc_g[rt][mt][2], pw * acc_g[rt][mt][3]};
         } else {
 #pragma unroll
           for (int v = 0; v < 4; ++v)
-            if (nc + v < N) o[v] = acc_g[rt][mt][v];
+            if (nc + v < N) o[v] = pw * acc_g[rt][mt][v];
         }
       }
     }
@@ -481,18 +454,18 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(
 template <int MT, int RT>
 static int launch_grouped(hipStream_t s, const void* x, const float* weight, const void* w_gate_up, const void* w_down,
                           void* act, float* out, const int32_t* ints, int max_tiles, int64_t tokens, int K, int F, int top,
-                          float gate_alpha, float limit, float up_shift) {
+                          float gate_alpha, float limit, float up_shift, int weight_on_output) {
   const int64_t pairs = tokens * top;
   const int32_t* sorted = ints;
   const int32_t* t_e = ints + pairs;
   const int32_t* t_f = t_e + max_tiles;
   const int32_t* t_c = t_f + max_tiles;
   moe_grouped_kernel<MT, RT, true><<<dim3(static_cast<unsigned>(ceil_div(F, 64 * RT)), static_cast<unsigned>(max_tiles)), dim3(256), 0, s>>>(
-      static_cast<const bf16_t*>(x), weight, static_cast<const bf16_t*>(w_gate_up), sorted, t_e, t_f, t_c,
+      static_cast<const bf16_t*>(x), weight_on_output ? nullptr : weight, static_cast<const bf16_t*>(w_gate_up), sorted, t_e, t_f, t_c,
       static_cast<bf16_t*>(act), nullptr, tokens, K, F, top, gate_alpha, limit, up_shift);
   if (check_launch("psamd_moe_experts_grouped (gate/up)")) return 1;
   moe_grouped_kernel<MT, RT, false><<<dim3(static_cast<unsigned>(ceil_div(K, 64 * RT)), static_cast<unsigned>(max_tiles)), dim3(256), 0, s>>>(
-      static_cast<const bf16_t*>(act), nullptr, static_cast<const bf16_t*>(w_down), sorted, t_e, t_f, t_c, nullptr, out,
+      static_cast<const bf16_t*>(act), weight_on_output ? weight : nullptr, static_cast<const bf16_t*>(w_down), sorted, t_e, t_f, t_c, nullptr, out,
       tokens, F, K, top, 0.f, 0.f, 0.f);
   return check_launch("psamd_moe_experts_grouped (down)");
 }
@@ -500,17 +473,33 @@ static int launch_grouped(hipStream_t s, const void* x, const float* weight, con
 template <typename A>
 static int launch_experts_rows(hipStream_t s, const void* x, const int32_t* chosen, const float* weight,
                                const void* w_gate_up, const void* w_down, void* act, float* out, int64_t tokens, int K,
-                               int F, int experts, int top, float gate_alpha, float limit, float up_shift) {
+                               int F, int experts, int top, float gate_alpha, float limit, float up_shift,
+                               int weight_on_output) {
   const unsigned pairs = static_cast<unsigned>(tokens * top);
   moe_gate_up_rows_kernel<A><<<dim3(pairs, static_cast<unsigned>(ceil_div(F, kRowsPerBlock))), dim3(256),
                                sizeof(float) * K, s>>>(
       static_cast<const A*>(x), chosen, weight, static_cast<const A*>(w_gate_up), static_cast<A*>(act), K, F, experts, top,
-      gate_alpha, limit, up_shift);
+      gate_alpha, limit, up_shift, weight_on_output);
   if (check_launch("psamd_moe_experts_rows (gate/up)")) return 1;
   moe_down_rows_kernel<A><<<dim3(pairs, static_cast<unsigned>(ceil_div(K, kRowsPerBlock))), dim3(256), sizeof(float) * F,
                             s>>>(static_cast<const A*>(act), chosen, static_cast<const A*>(w_down), out, tokens, K, F,
-                                 experts, top);
+                                 experts, top, weight_on_output ? weight : nullptr);
   return check_launch("psamd_moe_experts_rows (down)");
+}
+
+// out[t, :] *= sigmoid(x[t] . w): one number per token on the output of a branch every token takes.
+// One wave per token, the dot product in float.
+template <typename A>
+__global__ __launch_bounds__(256) void row_gate_kernel(float* __restrict__ out, const A* __restrict__ x,
+                                                       const float* __restrict__ w, int64_t tokens, int out_hidden, int hidden) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (t >= tokens) return;
+  float acc = 0.f;
+  for (int i = lane; i < hidden; i += kWave) acc = fmaf(to_float<A>(x[t * hidden + i]), w[i], acc);
+  const float g = 1.f / (1.f + expf(-wave_sum(acc)));
+  float* o = out + t * out_hidden;
+  for (int i = lane; i < out_hidden; i += kWave) o[i] *= g;
 }
 
 }  // namespace psamd
@@ -523,7 +512,8 @@ int psamd_moe_grouped_tile_rows(int64_t pairs, int experts);
 int psamd_moe_grouped_max_tiles(int64_t pairs, int experts);
 
 int psamd_moe_route(void* stream, const void* x, int x_dtype, const float* w_router, int32_t* chosen, float* weight,
-                    int64_t tokens, int K, int experts, int top) {
+                    int64_t tokens, int K, int experts, int top, const float* bias, int mode) {
+  PSAMD_REQUIRE(mode == 0 || mode == 1, "router mode 0 (sigmoid scores) or 1 (softmax over the chosen)");
   PSAMD_REQUIRE(tokens >= 0 && K > 0 && experts > 0 && top >= 1 && top <= experts, "bad sizes");
   PSAMD_REQUIRE(sizeof(float) * (static_cast<size_t>(K) + experts) <= 64 * 1024, "row and scores do not fit in LDS");
   PSAMD_REQUIRE(tokens <= 2147483647LL, "too many tokens for one launch");
@@ -533,10 +523,10 @@ int psamd_moe_route(void* stream, const void* x, int x_dtype, const float* w_rou
   const dim3 grid(static_cast<unsigned>(tokens));
   if (x_dtype == kBF16) {
     moe_route_kernel<bf16_t><<<grid, dim3(256), smem, s>>>(static_cast<const bf16_t*>(x), w_router, chosen, weight, K,
-                                                          experts, top);
+                                                          experts, top, bias, mode);
   } else if (x_dtype == kF32) {
     moe_route_kernel<float><<<grid, dim3(256), smem, s>>>(static_cast<const float*>(x), w_router, chosen, weight, K,
-                                                         experts, top);
+                                                         experts, top, bias, mode);
   } else {
     return fail("psamd_moe_route: x must be float32 or bfloat16");
   }
@@ -544,18 +534,20 @@ int psamd_moe_route(void* stream, const void* x, int x_dtype, const float* w_rou
 }
 
 int psamd_moe_topk(void* stream, const float* logits, int32_t* chosen, float* weight, int64_t tokens, int experts,
-                   int top) {
+                   int top, const float* bias, int mode) {
+  PSAMD_REQUIRE(mode == 0 || mode == 1, "router mode 0 (sigmoid scores) or 1 (softmax over the chosen)");
   PSAMD_REQUIRE(tokens >= 0 && experts > 0 && top >= 1 && top <= experts, "bad sizes");
   PSAMD_REQUIRE(sizeof(float) * 4 * static_cast<size_t>(experts) <= 64 * 1024, "scores do not fit in LDS");
   PSAMD_REQUIRE(ceil_div(tokens, 4) <= 2147483647LL, "too many tokens for one launch");
   if (tokens == 0) return 0;
   moe_topk_kernel<<<dim3(static_cast<unsigned>(ceil_div(tokens, 4))), dim3(256), sizeof(float) * 4 * experts,
-                    static_cast<hipStream_t>(stream)>>>(logits, chosen, weight, tokens, experts, top);
+                    static_cast<hipStream_t>(stream)>>>(logits, chosen, weight, tokens, experts, top, bias, mode);
   return check_launch("psamd_moe_topk");
 }
 
 int psamd_moe_topk_group(void* stream, const float* logits, int32_t* chosen, float* weight, int32_t* ints, int64_t tokens,
-                         int experts, int top) {
+                         int experts, int top, const float* bias, int mode) {
+  PSAMD_REQUIRE(mode == 0 || mode == 1, "router mode 0 (sigmoid scores) or 1 (softmax over the chosen)");
   PSAMD_REQUIRE(tokens >= 1 && tokens <= 64 && experts > 0 && experts <= 1024 && top >= 1 && top <= experts, "bad sizes");
   PSAMD_REQUIRE(ints != nullptr, "the grouping needs its integer scratch");
   const int64_t pairs = tokens * top;
@@ -564,14 +556,14 @@ int psamd_moe_topk_group(void* stream, const float* logits, int32_t* chosen, flo
   moe_topk_group_kernel<<<dim3(1), dim3(1024), sizeof(int32_t) * (4 * experts + 1) + sizeof(float) * 16 * experts,
                           static_cast<hipStream_t>(stream)>>>(logits, chosen, weight, static_cast<int>(tokens), experts, top, rows,
                                                               max_tiles, ints, ints + pairs, ints + pairs + max_tiles,
-                                                              ints + pairs + 2 * max_tiles);
+                                                              ints + pairs + 2 * max_tiles, bias, mode);
   return check_launch("psamd_moe_topk_group");
 }
 
 int psamd_moe_experts_rows(void* stream, const void* x, const int32_t* chosen, const float* weight,
                            const void* w_gate_up, const void* w_down, void* act, float* out, int dtype,
                            int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
-                           float up_shift) {
+                           float up_shift, int weight_on_output) {
   PSAMD_REQUIRE(tokens >= 0 && K > 0 && F > 0 && experts > 0 && top >= 1 && top <= experts, "bad sizes");
   PSAMD_REQUIRE(sizeof(float) * static_cast<size_t>(std::max(K, F)) <= 64 * 1024, "a row does not fit in LDS");
   PSAMD_REQUIRE(tokens * top <= 2147483647LL && ceil_div(std::max(K, F), kRowsPerBlock) <= 65535, "too large for one launch");
@@ -579,10 +571,10 @@ int psamd_moe_experts_rows(void* stream, const void* x, const int32_t* chosen, c
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == kBF16)
     return launch_experts_rows<bf16_t>(s, x, chosen, weight, w_gate_up, w_down, act, out, tokens, K, F, experts, top,
-                                       gate_alpha, limit, up_shift);
+                                       gate_alpha, limit, up_shift, weight_on_output);
   if (dtype == kF32)
     return launch_experts_rows<float>(s, x, chosen, weight, w_gate_up, w_down, act, out, tokens, K, F, experts, top,
-                                      gate_alpha, limit, up_shift);
+                                      gate_alpha, limit, up_shift, weight_on_output);
   return fail("psamd_moe_experts_rows: dtype must be float32 or bfloat16");
 }
 
@@ -603,7 +595,7 @@ int psamd_moe_grouped_max_tiles(int64_t pairs, int experts) {
 int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen, const float* weight,
                               const void* w_gate_up, const void* w_down, void* act, float* out, int32_t* ints,
                               int64_t tokens, int K, int F, int experts, int top, float gate_alpha, float limit,
-                              float up_shift, int grouped_already) {
+                              float up_shift, int grouped_already, int weight_on_output) {
   PSAMD_REQUIRE(tokens >= 0 && K > 0 && F > 0 && experts > 0 && top >= 1 && top <= experts, "bad sizes");
   PSAMD_REQUIRE(K % 8 == 0 && F % 8 == 0, "K and F must be multiples of 8");
   PSAMD_REQUIRE(experts <= 4096 && tokens * top <= (1 << 24), "too many experts or pairs");
@@ -622,12 +614,28 @@ int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen
   }
   if (rows == 128)
     return launch_grouped<8, 2>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha,
-                                limit, up_shift);
+                                limit, up_shift, weight_on_output);
   if (rows == 64)
     return launch_grouped<4, 2>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha,
-                                limit, up_shift);
+                                limit, up_shift, weight_on_output);
   return launch_grouped<1, 1>(s, x, weight, w_gate_up, w_down, act, out, ints, max_tiles, tokens, K, F, top, gate_alpha, limit,
-                              up_shift);
+                              up_shift, weight_on_output);
+}
+
+int psamd_row_gate(void* stream, float* out, const void* x, int act_dtype, const float* w, int64_t tokens, int out_hidden,
+                   int hidden) {
+  PSAMD_REQUIRE(tokens >= 0 && out_hidden > 0 && hidden > 0 && ceil_div(tokens, 4) <= 2147483647LL, "bad sizes");
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(ceil_div(tokens, 4)));
+  if (act_dtype == kBF16) {
+    row_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(out, static_cast<const bf16_t*>(x), w, tokens, out_hidden, hidden);
+  } else if (act_dtype == kF32) {
+    row_gate_kernel<float><<<grid, dim3(256), 0, s>>>(out, static_cast<const float*>(x), w, tokens, out_hidden, hidden);
+  } else {
+    return fail("psamd_row_gate: activation dtype must be float32 or bfloat16");
+  }
+  return check_launch("psamd_row_gate");
 }
 
 }  // extern "C"

@@ -77,7 +77,7 @@ _SIGNATURES = {
     "psamd_scaled_add_rmsnorm": [_vp, _vp, _f32, _vp, _i32, _i32, _i64, _vp, _i32, _f32, _vp, _i32, _i64, _i32],
     "psamd_to_activation": [_vp, _vp, _vp, _i32, _i64],
     "psamd_rope_norm_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _i32, _f32, _vp, _vp],
-    "psamd_qk_prepare_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _i32, _f32, _vp, _vp, _vp, _i32, _vp, _vp],
+    "psamd_qk_prepare_kv_append": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _i32, _f32, _vp, _vp, _vp, _i32, _vp, _vp, _i32],
     "psamd_residual_add": [_vp, _vp, _vp, _i32, _i32, _i64, _i64, _i32],
     "psamd_stream_affine": [_vp, _vp, _i64, _i32, _f32, _vp],
     "psamd_concat_to_activation": [_vp, _vp, _vp, _vp, _i32, _i64, _i32],
@@ -86,12 +86,22 @@ _SIGNATURES = {
     "psamd_causal_conv": [_vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _i32],
     "psamd_gated_scan": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _i32,
                          _vp, _i32, _i32, _vp, _i32, _vp, _i32, _i32, _i32],
-    "psamd_moe_route": [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
-    "psamd_moe_topk": [_vp, _vp, _vp, _vp, _i64, _i32, _i32],
+    "psamd_moe_route": [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp, _i32],
+    "psamd_moe_topk": [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _i32],
     "psamd_moe_grouped_max_tiles": [_i64, _i32],
-    "psamd_moe_experts_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32, _i32],
-    "psamd_moe_topk_group": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32],
-    "psamd_moe_experts_rows": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32],
+    "psamd_moe_experts_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32, _i32, _i32],
+    "psamd_moe_topk_group": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _i32],
+    "psamd_moe_experts_rows": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32, _i32],
+    "psamd_row_gate": [_vp, _vp, _vp, _i32, _vp, _i64, _i32, _i32],
+    "psamd_layernorm_step": [_vp, _vp, _vp, _vp, _i32, _i32, _i64, _vp, _vp, _f32, _vp, _vp, _f32, _vp, _i32, _i64, _i32],
+    "psamd_add_sinusoid": [_vp, _vp, _vp, _vp, _i64, _i32],
+    "psamd_short_conv": [_vp, _vp, _i32, _i64, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32],
+    "psamd_gated_delta_prepare": [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _i32, _f32, _f32],
+    "psamd_general_delta_prepare": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _i32, _i32,
+                                    _i32, _f32, _f32],
+    "psamd_delta_scan": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64,
+                         _vp, _vp, _i32, _i32, _i32, _i32, _i32],
+    "psamd_heads_norm_gate": [_vp, _vp, _i64, _i32, _i32, _vp, _i32, _f32, _vp, _i32, _i64, _i32, _vp],
 }
 
 
@@ -437,13 +447,15 @@ class HipOps:
                                                None if kv is None else write_slot.data_ptr()))
 
     def rope_norm_kv_append(self, qkv, hq: int, hkv: int, d: int, positions, table, kv, write_slot, norm_dim: int,
-                            norm_eps: float, bias=None, q_weight=None, k_weight=None, values_from_keys: bool = False) -> None:
+                            norm_eps: float, bias=None, q_weight=None, k_weight=None, values_from_keys: bool = False,
+                            q_weight_per_head: bool = False) -> None:
         """``rope_kv_append`` with every q and k head divided, behind the rotation, by the root mean
         square over its ``norm_dim`` own dimensions (0: no norm; the head's other slots hold zeros).
         ``hkv`` may be 0: rows of queries alone, nothing written to pages. ``bias`` (float32
         [(hq + hkv) * d]) is added to the q and k heads first; ``q_weight`` / ``k_weight`` (float32 [d])
         multiply the normalized heads; ``values_from_keys``: the rows are [q | k] only and the value
-        written to the pages is the key as projected (with its bias, before rotation and norm)."""
+        written to the pages is the key as projected (with its bias, before rotation and norm).
+        ``q_weight_per_head``: ``q_weight`` is float32 [hq * d], a factor of its own for every query head."""
         t = qkv.shape[0]
         general = bias is not None or q_weight is not None or k_weight is not None or values_from_keys
         if general:
@@ -451,7 +463,7 @@ class HipOps:
             self._need(qkv.shape[1] == row_heads * d and qkv.is_contiguous(), "rope_norm_kv_append: qkv shape")
             self._need(positions.dtype == torch.int32 and positions.numel() == t, "rope_norm_kv_append: positions")
             self._need(0 <= norm_dim <= d and d % 2 == 0 and d <= 256, "rope_norm_kv_append: head sizes")
-            for v, n in ((bias, (hq + hkv) * d), (q_weight, d), (k_weight, d)):
+            for v, n in ((bias, (hq + hkv) * d), (q_weight, hq * d if q_weight_per_head else d), (k_weight, d)):
                 if v is not None:
                     self._need(v.dtype == torch.float32 and v.numel() == n and v.is_contiguous(),
                                "rope_norm_kv_append: bias and norm weights are float32")
@@ -465,7 +477,7 @@ class HipOps:
             self._ok(self.lib.psamd_qk_prepare_kv_append(
                 self._stream(), qkv.data_ptr(), _code(qkv.dtype), t, hq, hkv, d, positions.data_ptr(), _ptr(table),
                 int(norm_dim), float(norm_eps), _ptr(bias), _ptr(q_weight), _ptr(k_weight), int(values_from_keys), _ptr(kv),
-                None if kv is None else write_slot.data_ptr()))
+                None if kv is None else write_slot.data_ptr(), int(q_weight_per_head)))
             return
         self._need(qkv.shape[1] == (hq + 2 * hkv) * d and qkv.is_contiguous(), "rope_norm_kv_append: qkv shape")
         self._need(positions.dtype == torch.int32 and positions.numel() == t, "rope_norm_kv_append: positions")
@@ -644,14 +656,19 @@ class HipOps:
 
     # ------------------------------------------------------------------ experts
 
-    def moe_route(self, x, w_router, chosen, weight, w_router_act=None) -> None:
+    def moe_route(self, x, w_router, chosen, weight, w_router_act=None, bias=None, mode: int = 0) -> None:
         """chosen[t, :], weight[t, :] = the experts with the largest sigmoid(x[t] . w_router[e]) and
         those scores, largest first, the lower index among equals; scores in 32-bit. With the router
         also given in the activation dtype (``w_router_act``), a step of more than
         ``MOE_ROUTE_FUSED_MAX_TOKENS`` tokens takes its logits from the product kernels (float32 sums of
         exact products, float32 out) and the choice from a kernel of its own: the fused kernel reads
         the whole router once per token with one workgroup (8 tokens of a 32 x 2,048 router: 94 us
-        against 5 + 4 for product and choice), so the bound is 0 and it serves callers without that copy."""
+        against 5 + 4 for product and choice), so the bound is 0 and it serves callers without that copy.
+        ``bias`` (float32 [E]) is added to the logits; ``mode`` 1: the largest logits are chosen and the
+        weights are the softmax over the chosen logits alone."""
+        if bias is not None:
+            self._need(bias.dtype == torch.float32 and bias.numel() == w_router.shape[0] and bias.is_contiguous(),
+                       "moe_route: the bias is float32 [E]")
         t, k = x.shape
         e, top = w_router.shape[0], chosen.shape[1]
         if (w_router_act is not None and t > self.MOE_ROUTE_FUSED_MAX_TOKENS and w_router_act.dtype == x.dtype
@@ -666,10 +683,11 @@ class HipOps:
                 # A small step: the workgroup that chooses also sorts the pairs for the experts' kernels.
                 ints = self._group_ints(t, top, e)
                 self._ok(self.lib.psamd_moe_topk_group(self._stream(), logits.data_ptr(), chosen.data_ptr(), weight.data_ptr(),
-                                                       ints.data_ptr(), t, e, top))
+                                                       ints.data_ptr(), t, e, top, _ptr(bias), int(mode)))
                 self._grouped_for = (chosen.data_ptr(), t, top, e)
                 return
-            self._ok(self.lib.psamd_moe_topk(self._stream(), logits.data_ptr(), chosen.data_ptr(), weight.data_ptr(), t, e, top))
+            self._ok(self.lib.psamd_moe_topk(self._stream(), logits.data_ptr(), chosen.data_ptr(), weight.data_ptr(), t, e, top,
+                                             _ptr(bias), int(mode)))
             return
         self._grouped_for = None
         self._need(x.is_contiguous() and w_router.dtype == torch.float32 and w_router.is_contiguous()
@@ -678,7 +696,7 @@ class HipOps:
                    and weight.shape == (t, top) and chosen.is_contiguous() and weight.is_contiguous() and 1 <= top <= e,
                    "moe_route: outputs must be int32 and float32 [T, top]")
         self._ok(self.lib.psamd_moe_route(self._stream(), x.data_ptr(), _code(x.dtype), w_router.data_ptr(),
-                                          chosen.data_ptr(), weight.data_ptr(), t, k, e, top))
+                                          chosen.data_ptr(), weight.data_ptr(), t, k, e, top, _ptr(bias), int(mode)))
 
     def _groups_pairs(self, dtype: torch.dtype, t: int, k: int) -> bool:
         """Whether a step of ``t`` tokens of width ``k`` runs its experts grouped by expert."""
@@ -689,9 +707,10 @@ class HipOps:
         return self.ws.get("moe.group", (t * top + 3 * tiles,), torch.int32)
 
     def moe_experts(self, x, chosen, weight, w_gate_up, w_down, act, out, gate_alpha: float, limit: float,
-                    up_shift: float) -> None:
+                    up_shift: float, weight_on_output: bool = False) -> None:
         """out[j, t] = down_e(act_e(weight[t, j] * x[t])) for e = chosen[t, j], as float32 slices [top, T, K];
-        ``act`` [T * top, F] is scratch in the activation dtype."""
+        ``act`` [T * top, F] is scratch in the activation dtype. ``weight_on_output``: out[j, t] =
+        weight[t, j] * down_e(act_e(x[t])) instead."""
         t, k = x.shape
         top = chosen.shape[1]
         e, f2, _ = w_gate_up.shape
@@ -712,12 +731,176 @@ class HipOps:
             self._ok(self.lib.psamd_moe_experts_grouped(self._stream(), x.data_ptr(), chosen.data_ptr(), weight.data_ptr(),
                                                         w_gate_up.data_ptr(), w_down.data_ptr(), act.data_ptr(),
                                                         out.data_ptr(), ints.data_ptr(), t, k, f, e, top, float(gate_alpha),
-                                                        float(limit), float(up_shift), done))
+                                                        float(limit), float(up_shift), done, int(weight_on_output)))
             return
         self._ok(self.lib.psamd_moe_experts_rows(self._stream(), x.data_ptr(), chosen.data_ptr(), weight.data_ptr(),
                                                  w_gate_up.data_ptr(), w_down.data_ptr(), act.data_ptr(), out.data_ptr(),
                                                  _code(x.dtype), t, k, f, e, top, float(gate_alpha), float(limit),
-                                                 float(up_shift)))
+                                                 float(up_shift), int(weight_on_output)))
+
+    def row_gate(self, out, x, w) -> None:
+        """out[t, :] *= sigmoid(x[t] . w): float32 out [T, N], x [T, K] in a kernel dtype, w float32 [K]."""
+        t, k = x.shape
+        self._need(out.dtype == torch.float32 and out.is_contiguous() and out.shape[0] == t and x.is_contiguous()
+                   and w.dtype == torch.float32 and w.numel() == k and w.is_contiguous(), "row_gate: operands")
+        self._ok(self.lib.psamd_row_gate(self._stream(), out.data_ptr(), x.data_ptr(), _code(x.dtype), w.data_ptr(), t,
+                                         out.shape[1], k))
+
+    # ------------------------------------------------------- layer norm, sinusoid
+
+    def layernorm_step(self, residual, delta, post, pre, out, rows=None) -> None:
+        """Layer norm with weight and bias around the stream; ``post`` and ``pre`` are (weight, bias, eps)
+        with float32 [H] tensors, or None. With ``delta`` ([T, H] in a kernel dtype or [S, T, H] float32
+        slices): residual += post(delta). With ``out``: out = pre(residual) in out's dtype; ``rows``
+        (int32 [n], without a delta) picks the rows of the stream that ``out`` is made of."""
+        t, h = residual.shape
+        self._need(residual.dtype == torch.float32 and residual.is_contiguous(), "layernorm_step: the stream is float32")
+        for terms in (post, pre):
+            if terms is not None:
+                self._need(all(v.dtype == torch.float32 and v.numel() == h and v.is_contiguous() for v in terms[:2]),
+                           "layernorm_step: weight and bias are float32 [H]")
+        self._need((delta is None) == (post is None) and (out is None) == (pre is None) and (delta is not None or out is not None),
+                   "layernorm_step: a delta with the norm behind it, an output with the norm in front of it")
+        n = t
+        if rows is not None:
+            self._need(delta is None and rows.dtype == torch.int32 and rows.is_contiguous(), "layernorm_step: rows are int32, without a delta")
+            n = rows.numel()
+        dptr, dcode, slices, stride = self._delta_args(delta, t, h, delta.dtype if delta is not None else torch.float32)
+        if out is not None:
+            self._need(out.shape == (n, h) and out.is_contiguous(), "layernorm_step: bad output shape")
+        pw, pb, pe = (post[0].data_ptr(), post[1].data_ptr(), float(post[2])) if post is not None else (None, None, 0.0)
+        qw, qb, qe = (pre[0].data_ptr(), pre[1].data_ptr(), float(pre[2])) if pre is not None else (None, None, 0.0)
+        self._ok(self.lib.psamd_layernorm_step(self._stream(), residual.data_ptr(), _ptr(rows), dptr, dcode, max(slices, 1), stride,
+                                               pw, pb, pe, qw, qb, qe, _ptr(out), _code(out.dtype) if out is not None else _F32,
+                                               n, h))
+
+    def add_sinusoid(self, x, positions, freq) -> None:
+        """x[t, 2i] += sin(positions[t] * freq[i]), x[t, 2i + 1] += cos(.); x float32 [T, H], freq float64 [(H + 1) // 2]."""
+        t, h = x.shape
+        self._need(x.dtype == torch.float32 and x.is_contiguous() and positions.dtype == torch.int32 and positions.numel() == t
+                   and freq.dtype == torch.float64 and freq.numel() == (h + 1) // 2 and freq.is_contiguous(), "add_sinusoid: operands")
+        self._ok(self.lib.psamd_add_sinusoid(self._stream(), x.data_ptr(), positions.data_ptr(), freq.data_ptr(), t, h))
+
+    # ------------------------------------------------------------ delta rules
+
+    def short_conv(self, rows, col: int, conv_w, out, state, state_offset: int, ctx, silu: bool = True) -> None:
+        """out[t, c] = act(sum_j conv_w[c, j] v(t - (taps - 1) + j, c)), v = rows[:, col + c], over each item's
+        tokens, continued in front of an item's first token from the inputs its state slot saved
+        (``state[slot, state_offset + j * channels + c]``, oldest first), which are then replaced by the
+        item's last taps - 1 inputs. ``out`` is float32 [T, channels]."""
+        t, channels = out.shape
+        taps = conv_w.shape[1]
+        self._need(rows.is_contiguous() and rows.shape[0] == t and 0 <= col and col + channels <= rows.shape[1], "short_conv: rows")
+        self._need(out.dtype == torch.float32 and out.is_contiguous() and conv_w.dtype == torch.float32
+                   and tuple(conv_w.shape) == (channels, taps) and conv_w.is_contiguous(), "short_conv: float32 taps [channels, taps] and output")
+        self._need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
+                   and 0 <= state_offset and state_offset + (taps - 1) * channels <= state.shape[1], "short_conv: the state's saved inputs")
+        self._need(t == ctx.num_tokens, "short_conv: token count differs from the step batch")
+        self._ok(self.lib.psamd_short_conv(self._stream(), rows.data_ptr() + col * rows.element_size(), _code(rows.dtype),
+                                           rows.shape[1], conv_w.data_ptr(), out.data_ptr(), channels,
+                                           state.data_ptr() + 4 * state_offset, state.shape[1], ctx.tok_item.data_ptr(),
+                                           ctx.item_start.data_ptr(), ctx.slots.data_ptr(), t, ctx.num_items, channels, taps,
+                                           int(silu)))
+
+    def gated_delta_prepare(self, u, groups: int, dim: int, gates, decay_log, decay_bias, coef, q_scale: float,
+                            unit_eps: float) -> None:
+        """u (float32 [T, >= 2 groups dim]) starts with the query and key vectors ([groups, dim] each): each is
+        divided by sqrt(sum of squares + unit_eps) in place, the queries also times q_scale. gates float32
+        [T, 2 heads] = [strength logits | decay inputs] -> coef float32 [T, 3 heads] = [g | -b | b] with
+        b = sigmoid(.), g = exp(-exp(decay_log[h]) softplus(. + decay_bias[h]))."""
+        t = u.shape[0]
+        heads = decay_log.numel()
+        self._need(u.dtype == torch.float32 and u.is_contiguous() and u.shape[1] >= 2 * groups * dim, "gated_delta_prepare: u")
+        self._need(gates.dtype == torch.float32 and gates.shape == (t, 2 * heads) and gates.is_contiguous()
+                   and coef.dtype == torch.float32 and coef.shape == (t, 3 * heads) and coef.is_contiguous(),
+                   "gated_delta_prepare: gates [T, 2 heads] and coef [T, 3 heads] are float32")
+        for v in (decay_log, decay_bias):
+            self._need(v.dtype == torch.float32 and v.numel() == heads and v.is_contiguous(), "gated_delta_prepare: float32 [heads]")
+        self._ok(self.lib.psamd_gated_delta_prepare(self._stream(), u.data_ptr(), u.shape[1], groups, dim, gates.data_ptr(),
+                                                    decay_log.data_ptr(), decay_bias.data_ptr(), coef.data_ptr(), t, heads,
+                                                    float(q_scale), float(unit_eps)))
+
+    def general_delta_prepare(self, rows, r_col: int, k_col: int, v_col: int, a_col: int, l_col: int, rate_bias, decay_out,
+                              decay_bias, operands, heads: int, dim: int, decay_floor: float, unit_eps: float) -> None:
+        """From rows (a kernel dtype; r, k, v and the rate's logits [heads, dim] at their columns, the decay
+        map's inner values [rank] at l_col) to operands float32 [T, 6 heads dim] = [r | k | v | w | p | c]:
+        w = exp(-decay_floor sigmoid(decay_out tanh(l) + decay_bias)), c = k / sqrt(sum k^2 + unit_eps) per head,
+        p = -sigmoid(rate logits + rate_bias) * c."""
+        t = rows.shape[0]
+        hd = heads * dim
+        rank = decay_out.shape[1]
+        self._need(rows.is_contiguous() and max(r_col, k_col, v_col, a_col) + hd <= rows.shape[1] and l_col + rank <= rows.shape[1]
+                   and min(r_col, k_col, v_col, a_col, l_col) >= 0, "general_delta_prepare: columns outside the rows")
+        self._need(operands.dtype == torch.float32 and operands.shape == (t, 6 * hd) and operands.is_contiguous(),
+                   "general_delta_prepare: operands are float32 [T, 6 heads dim]")
+        for v, shape in ((rate_bias, (hd,)), (decay_out, (hd, rank)), (decay_bias, (hd,))):
+            self._need(v.dtype == torch.float32 and tuple(v.shape) == shape and v.is_contiguous(), "general_delta_prepare: float32 parameters")
+        self._ok(self.lib.psamd_general_delta_prepare(self._stream(), rows.data_ptr(), _code(rows.dtype), rows.shape[1], r_col, k_col,
+                                                      v_col, a_col, l_col, rate_bias.data_ptr(), decay_out.data_ptr(),
+                                                      decay_bias.data_ptr(), operands.data_ptr(), t, heads, dim, rank,
+                                                      float(decay_floor), float(unit_eps)))
+
+    def delta_scan(self, keys, directions, removals, queries, key_groups: int, decay_vectors, decay, removal_scale,
+                   value_scale, values, out, state, state_offset: int, ctx, heads: int, dim: int, vdim: int,
+                   reads_decayed: bool) -> None:
+        """The delta-rule recurrence over each item's tokens from its state slot. Every operand is a pair
+        (float32 tensor [T, row], first column) or None. Per head h (its key group g = h // (heads / key_groups))
+        and token: S' = d S with d = decay_vectors[h, :] (per key channel) times decay[h] (a number), either may
+        be None = 1; S = S' + (removal_scale[h] removals[g]) (directions[g]^T S*) + keys[g] (value_scale[h]
+        values[h])^T with S* = S' if ``reads_decayed`` else the S before the token; out[h] = S^T queries[g].
+        ``keys``, ``directions``, ``removals``, ``queries`` lie in one tensor, as do ``decay``, ``removal_scale``,
+        ``value_scale``. The state of head h is ``state[slot, state_offset + (h vdim + j) dim + i]``; out is
+        float32 [T, heads vdim]."""
+        t = out.shape[0]
+        self._need(t == ctx.num_tokens and out.dtype == torch.float32 and out.shape == (t, heads * vdim) and out.is_contiguous(),
+                   "delta_scan: out is float32 [T, heads vdim]")
+        self._need(heads % key_groups == 0 and 1 <= dim <= 256 and vdim >= 1, "delta_scan: sizes")
+        base = keys[0]
+        for pair in (keys, directions, removals, queries):
+            self._need(pair[0] is base and 0 <= pair[1] and pair[1] + key_groups * dim <= base.shape[1], "delta_scan: key-side operands share a tensor")
+        self._need(base.dtype == torch.float32 and base.is_contiguous() and base.shape[0] == t, "delta_scan: float32 operands")
+        scal = [p for p in (decay, removal_scale, value_scale) if p is not None]
+        sbase = scal[0][0] if scal else None
+        for pair in scal:
+            self._need(pair[0] is sbase and 0 <= pair[1] and pair[1] + heads <= sbase.shape[1], "delta_scan: the numbers per head share a tensor")
+        if sbase is not None:
+            self._need(sbase.dtype == torch.float32 and sbase.is_contiguous() and sbase.shape[0] == t, "delta_scan: float32 numbers per head")
+        if decay_vectors is not None:
+            dv = decay_vectors[0]
+            self._need(dv.dtype == torch.float32 and dv.is_contiguous() and dv.shape[0] == t and 0 <= decay_vectors[1]
+                       and decay_vectors[1] + heads * dim <= dv.shape[1], "delta_scan: decay vectors")
+        xv = values[0]
+        self._need(xv.dtype == torch.float32 and xv.is_contiguous() and xv.shape[0] == t and 0 <= values[1]
+                   and values[1] + heads * vdim <= xv.shape[1], "delta_scan: values")
+        self._need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous() and 0 <= state_offset
+                   and state_offset + heads * dim * vdim <= state.shape[1], "delta_scan: the state")
+
+        def at(pair):
+            return None if pair is None else pair[0].data_ptr() + 4 * pair[1]
+
+        self._ok(self.lib.psamd_delta_scan(
+            self._stream(), at(keys), at(directions), at(removals), at(queries), base.shape[1], key_groups,
+            at(decay_vectors), 0 if decay_vectors is None else decay_vectors[0].shape[1], at(decay), at(removal_scale),
+            at(value_scale), 0 if sbase is None else sbase.shape[1], at(values), xv.shape[1], out.data_ptr(), out.shape[1],
+            state.data_ptr() + 4 * state_offset, state.shape[1], ctx.item_start.data_ptr(), ctx.slots.data_ptr(),
+            ctx.num_items, heads, dim, vdim, int(reads_decayed)))
+
+    def heads_norm_gate(self, o, heads: int, vdim: int, weight, weight_per_head: bool, eps: float, gate_rows, gate_col: int,
+                        activation: str, out) -> None:
+        """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight * act(gate[t, h, :]): o float32
+        [T, heads vdim]; weight float32 [vdim] shared by the heads, or [heads vdim]; the gate lies in
+        ``gate_rows`` (a kernel dtype) from column ``gate_col``; act "silu" or "sigmoid"; out in that dtype."""
+        t = o.shape[0]
+        self._need(o.dtype == torch.float32 and o.shape == (t, heads * vdim) and o.is_contiguous(), "heads_norm_gate: o is float32")
+        self._need(weight.dtype == torch.float32 and weight.numel() == (heads * vdim if weight_per_head else vdim)
+                   and weight.is_contiguous(), "heads_norm_gate: weight")
+        self._need(gate_rows.is_contiguous() and gate_rows.shape[0] == t and 0 <= gate_col
+                   and gate_col + heads * vdim <= gate_rows.shape[1], "heads_norm_gate: the gate's columns")
+        self._need(out.dtype == gate_rows.dtype and out.shape == (t, heads * vdim) and out.is_contiguous(), "heads_norm_gate: out")
+        self._ok(self.lib.psamd_heads_norm_gate(self._stream(), o.data_ptr(), t, heads, vdim, weight.data_ptr(), int(weight_per_head),
+                                                float(eps), gate_rows.data_ptr() + gate_col * gate_rows.element_size(),
+                                                _code(gate_rows.dtype), gate_rows.shape[1], {"silu": 0, "sigmoid": 1}[activation],
+                                                out.data_ptr()))
 
     # --------------------------------------------------------------- attention
 

@@ -103,14 +103,17 @@ class PagedAttention(Mixer):
     * ``sink``: a learned number per head (name "sink") whose exponential joins the softmax's
       denominator; it has no key and no value.
     * ``distance_bias`` = {"buckets": B, "far": D}: a learned table [B, heads] (name "rel") whose
-      row bucket(i - j) is added to the scaled score of query i and key j (``distance_bucket``)."""
+      row bucket(i - j) is added to the scaled score of query i and key j (``distance_bucket``).
+    * ``head_scale``: a learned number per query head (name "head_scale") that multiplies the head's
+      scores beside ``scale``. It is folded, in 32-bit, into the factor each query head is multiplied
+      with behind its norm (a weight per head instead of one shared by the heads)."""
 
     def __init__(self, hidden_size: int, positions: Mapping[str, PositionEncoding], num_heads: int,
                  num_kv_heads: int, head_dim: int, names: Mapping[str, str], position: str | None = None,
                  window: int | None = None, scale: float | None = None, value_dim: int | None = None,
                  qk_norm_eps: float | None = None, own_kv: bool = True, exact_weights: bool = False,
                  qk_bias: bool = False, qk_norm_weights: bool = False, values_are_keys: bool = False,
-                 sink: bool = False, distance_bias: Mapping[str, Any] | None = None) -> None:
+                 sink: bool = False, distance_bias: Mapping[str, Any] | None = None, head_scale: bool = False) -> None:
         if num_kv_heads < 1 or num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads not divisible by {num_kv_heads} kv heads")
         self.hidden_size = int(hidden_size)
@@ -121,17 +124,18 @@ class PagedAttention(Mixer):
         self.exact_weights = bool(exact_weights)
         self.qk_bias, self.qk_norm_weights = bool(qk_bias), bool(qk_norm_weights)
         self.values_are_keys, self.has_sink = bool(values_are_keys), bool(sink)
+        self.head_scale = bool(head_scale)
         self.distance_bias = None if distance_bias is None else (int(distance_bias["buckets"]), float(distance_bias["far"]))
         if self.qk_norm_weights and self.qk_norm_eps is None:
             raise ValueError("weights on the q/k norm need qk_norm_eps")
         if self.values_are_keys and (self.value_dim != self.head_dim or not self.own_kv):
             raise ValueError("values that are the keys have the keys' size and belong to a layer with keys of its own")
-        if (self.qk_bias or self.qk_norm_weights) and not self.own_kv:
-            raise ValueError("biases and norm weights on q and k are implemented for layers with keys of their own")
+        if self.qk_bias and not self.own_kv:
+            raise ValueError("biases on q and k are implemented for layers with keys of their own")
         if self.distance_bias is not None and not 2 <= self.distance_bias[0] < 2 * self.distance_bias[1]:
             raise ValueError(f"a distance bias needs at least 2 buckets and a reach beyond half of them, got {self.distance_bias}")
         extras = (self.qk_bias or self.qk_norm_weights or self.values_are_keys or self.has_sink
-                  or self.distance_bias is not None)
+                  or self.distance_bias is not None or self.head_scale)
         self.bias = self.q_norm_weight = self.k_norm_weight = self.sink = self.distance_table = None
         self.names = dict(names)
         self.window = None if window is None else int(window)
@@ -173,7 +177,10 @@ class PagedAttention(Mixer):
             want[n["k_bias"]] = WeightWant((self.num_kv_heads * self.head_dim,), "bias")
         if self.qk_norm_weights:
             want[n["q_norm"]] = WeightWant((self.head_dim,), "norm")
-            want[n["k_norm"]] = WeightWant((self.head_dim,), "norm")
+            if self.own_kv:                  # a layer that reads another layer's keys reads them as normed there
+                want[n["k_norm"]] = WeightWant((self.head_dim,), "norm")
+        if self.head_scale:
+            want[n["head_scale"]] = WeightWant((self.num_heads,), "norm")
         if self.has_sink:
             want[n["sink"]] = WeightWant((self.num_heads,), "bias")
         if self.distance_bias is not None:
@@ -220,9 +227,18 @@ class PagedAttention(Mixer):
             both = [self._spread(tensors[n[key]].to(torch.float32)[:, None], heads, self.head_dim, self.index)
                     for key, heads in (("q_bias", self.num_heads), ("k_bias", self.num_kv_heads))]
             self.bias = on_device(torch.cat(both, dim=0).view(-1))
+        self.q_weight_per_head = False
         if self.qk_norm_weights:
             self.q_norm_weight = on_device(self._spread(tensors[n["q_norm"]].to(torch.float32)[:, None], 1, self.head_dim, self.index).view(-1))
-            self.k_norm_weight = on_device(self._spread(tensors[n["k_norm"]].to(torch.float32)[:, None], 1, self.head_dim, self.index).view(-1))
+            if self.own_kv:
+                self.k_norm_weight = on_device(self._spread(tensors[n["k_norm"]].to(torch.float32)[:, None], 1, self.head_dim, self.index).view(-1))
+        if self.head_scale:
+            # score = scale * number[h] * q.k: the number goes into the query head's factor, [heads, slots].
+            per_head = tensors[n["head_scale"]].to(torch.float32).view(-1, 1)
+            shared = self.q_norm_weight.cpu() if self.q_norm_weight is not None else \
+                self._spread(torch.ones((self.head_dim, 1)), 1, self.head_dim, self.index).view(-1)
+            self.q_norm_weight = on_device((per_head * shared[None, :]).reshape(-1))
+            self.q_weight_per_head = True
         if self.has_sink:
             self.sink = on_device(tensors[n["sink"]])
         if self.distance_bias is not None:
@@ -250,7 +266,13 @@ class PagedAttention(Mixer):
             qkv = ws.get("attn.qkv" if own else "attn.q", (t, self.row_width), rt.dtype)
             ops.linear(x, self.w_qkv, qkv)
             norm_dim, eps = (self.head_dim, self.qk_norm_eps) if self.qk_norm_eps is not None else (0, 0.0)
-            if self.qk_bias or self.qk_norm_weights or self.values_are_keys:
+            if self.head_scale:
+                ops.rope_norm_kv_append(qkv, self.num_heads, own, self.slots, ctx.positions, table,
+                                        cache.kv if writes_cache else None, ctx.groups[cache.group].write_slot,
+                                        norm_dim, eps, bias=self.bias, q_weight=self.q_norm_weight,
+                                        k_weight=self.k_norm_weight, values_from_keys=self.values_are_keys,
+                                        q_weight_per_head=self.q_weight_per_head)
+            elif self.qk_bias or self.qk_norm_weights or self.values_are_keys:
                 ops.rope_norm_kv_append(qkv, self.num_heads, own, self.slots, ctx.positions, table,
                                         cache.kv if writes_cache else None, ctx.groups[cache.group].write_slot,
                                         norm_dim, eps, bias=self.bias, q_weight=self.q_norm_weight,

@@ -121,6 +121,51 @@ class ParallelBlock:
         return self.feed_forward.forward(h, ctx)
 
 
+class SandwichBlock:
+    """A norm in front of and behind each sub-layer: x <- x + post1(mixer(pre1(x))), then, when the
+    layer has a feed-forward, x <- x + post2(feed_forward(pre2(x))).
+
+    The sub-layers hand their output back (``ctx.residual`` is None while they run): it is
+    normalized before it is added. The norm behind the mixer and the norm in front of the
+    feed-forward are one kernel (``add_normed`` of the norms). The stream is complete when the
+    block returns; nothing is left pending. ``mixer_post_norm`` / ``feed_forward_post_norm`` come
+    from ``LayerSpec.extra_norms``."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward | None, mixer_norm: Norm, feed_forward_norm: Norm | None,
+                 mixer_post_norm: Norm, feed_forward_post_norm: Norm | None = None) -> None:
+        if (feed_forward is None) != (feed_forward_norm is None) or (feed_forward is None) != (feed_forward_post_norm is None):
+            raise ValueError("a feed-forward comes with its two norms, a layer without one has neither")
+        for norm in (mixer_post_norm, feed_forward_post_norm):
+            if norm is not None and not hasattr(norm, "add_normed"):
+                raise ValueError("the norm behind a sub-layer must offer add_normed")
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+        self.mixer_post_norm, self.feed_forward_post_norm = mixer_post_norm, feed_forward_post_norm
+
+    def parts(self) -> list[Part]:
+        out = [self.mixer_norm, self.mixer, self.mixer_post_norm]
+        if self.feed_forward is not None:
+            out += [self.feed_forward_norm, self.feed_forward, self.feed_forward_post_norm]
+        return out
+
+    def forward(self, residual: torch.Tensor, pending: torch.Tensor | None, ctx: "StepContext", cache: Any,
+                state: torch.Tensor | None, writes_cache: bool) -> None:
+        ctx.stream_copy = None
+        h = self.mixer_norm.add_norm(residual, pending, "block.x")
+        kept, ctx.residual = ctx.residual, None          # the sub-layers hand their output back: it is normalized first
+        try:
+            mixed = self.mixer.forward(h, ctx, cache, state, writes_cache)
+            if self.feed_forward is None:
+                self.mixer_post_norm.add_normed(residual, mixed)
+            else:
+                h = self.mixer_post_norm.add_normed(residual, mixed, then=self.feed_forward_norm, out_name="block.x")
+                self.feed_forward_post_norm.add_normed(residual, self.feed_forward.forward(h, ctx))
+        finally:
+            ctx.residual = kept
+        return None
+
+
 register_block("prenorm", PreNormBlock)
+register_block("sandwich", SandwichBlock)
 register_block("parallel", ParallelBlock)
 register_block("postnorm", PostNormBlock)

@@ -10,6 +10,7 @@ import torch
 
 from . import attention as _attention  # noqa: F401  (registers the built-in parts)
 from . import block as _block  # noqa: F401
+from . import delta as _delta  # noqa: F401
 from . import latent as _latent  # noqa: F401
 from . import mlp as _mlp  # noqa: F401
 from . import moe as _moe  # noqa: F401

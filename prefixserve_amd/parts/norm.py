@@ -69,4 +69,60 @@ class RMSNorm(Norm):
         return residual if out is None else out
 
 
+class LayerNorm(Norm):
+    """(x - mean) / sqrt(mean((x - mean)^2) + eps) * weight + bias, eps inside the root; sums,
+    statistics and the residual sum in 32-bit, weight and bias widened to 32-bit once.
+
+    Beside the interface every norm has it offers ``add_normed``: the norm *behind* a sub-layer,
+    stream += norm(delta), fused with the norm in front of the next sub-layer where there is one.
+    ``name`` / ``bias_name``: the two tensors' names."""
+
+    def __init__(self, hidden_size: int, eps: float, name: str = "weight", bias_name: str | None = None) -> None:
+        self.hidden_size = int(hidden_size)
+        self.eps = float(eps)
+        self.name = name
+        self.bias_name = bias_name if bias_name is not None else name + ".b"
+
+    def weights(self) -> dict[str, WeightWant]:
+        return {self.name: WeightWant((self.hidden_size,), "norm"), self.bias_name: WeightWant((self.hidden_size,), "bias")}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        super().bind(tensors, rt)
+        self.weight = tensors[self.name].to(device=rt.device, dtype=torch.float32).contiguous()
+        self.bias = tensors[self.bias_name].to(device=rt.device, dtype=torch.float32).contiguous()
+        self.terms = (self.weight, self.bias, self.eps)          # what the kernel takes for one norm
+
+    def weight_bytes(self) -> int:
+        return 4 * (self.weight.numel() + self.bias.numel())
+
+    def add_norm(self, residual: torch.Tensor, delta: torch.Tensor | None, out_name: str,
+                 lazy: bool = False) -> torch.Tensor:
+        rt = self.rt
+        if delta is not None:
+            rt.ops.residual_add(residual, delta)
+        out = rt.workspace.get(out_name, (residual.shape[0], self.hidden_size), rt.dtype)
+        rt.ops.layernorm_step(residual, None, None, self.terms, out)
+        return out
+
+    def add_norm_rows(self, residual: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor,
+                      out_name: str, lazy: bool = False) -> torch.Tensor:
+        rt = self.rt
+        if delta is not None:
+            rt.ops.residual_add(residual, delta)
+        out = rt.workspace.get(out_name, (rows.shape[0], self.hidden_size), rt.dtype)
+        rt.ops.layernorm_step(residual, None, None, self.terms, out, rows=rows)
+        return out
+
+    def add_normed(self, residual: torch.Tensor, delta: torch.Tensor, then: "LayerNorm | None" = None,
+                   out_name: str = "block.x") -> torch.Tensor | None:
+        """residual (float32 [T,H], in place) += self(delta), where ``delta`` is [T,H] in the
+        activation dtype or [S,T,H] float32 slices that are summed first. With ``then``, another
+        norm of this kind, returns then(residual) in the activation dtype from the same kernel."""
+        rt = self.rt
+        out = None if then is None else rt.workspace.get(out_name, (residual.shape[0], self.hidden_size), rt.dtype)
+        rt.ops.layernorm_step(residual, delta, self.terms, None if then is None else then.terms, out)
+        return out
+
+
 register_norm("rmsnorm", RMSNorm)
+register_norm("layernorm", LayerNorm)

@@ -59,5 +59,26 @@ class StreamReentry(Transform):
         ops.stream_affine(t, 1.0, self.steps[ctx.pass_index])
 
 
+class SinusoidalPositions(Transform):
+    """t[row, 2i] += sin(p f_i), t[row, 2i + 1] += cos(p f_i) with f_i = base^(-2i / hidden) and p the
+    row's position: the fixed table of sines added to the token table's rows. The frequencies are
+    formed in float64 once; the kernel multiplies and reduces the angle in double before the 32-bit
+    sine, so far positions keep their digits. No weights."""
+
+    def __init__(self, hidden_size: int, vocab_size: int, base: float = 10000.0) -> None:
+        self.hidden_size, self.base = int(hidden_size), float(base)
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        super().bind(tensors, rt)
+        i = torch.arange((self.hidden_size + 1) // 2, dtype=torch.float64)
+        self.freq = torch.pow(torch.tensor(self.base, dtype=torch.float64), -2.0 * i / self.hidden_size).to(rt.device).contiguous()
+
+    def apply(self, t: torch.Tensor, ctx: "StepContext", rows: torch.Tensor | None) -> None:
+        if rows is not None:
+            raise ValueError("the sinusoid is added to the whole stream, row by row in order")
+        self.rt.ops.add_sinusoid(t, ctx.positions, self.freq)
+
+
 register_transform("scale", ScaleStream)
+register_transform("sinusoidal_positions", SinusoidalPositions)
 register_transform("reentry", StreamReentry)

@@ -185,7 +185,7 @@ class EmulatedOps:
             out.copy_(y.to(out.dtype))
 
     def rope_norm_kv_append(self, qkv, hq, hkv, d, positions, table, kv, write_slot, norm_dim, norm_eps, bias=None,
-                            q_weight=None, k_weight=None, values_from_keys=False) -> None:
+                            q_weight=None, k_weight=None, values_from_keys=False, q_weight_per_head=False) -> None:
         t = qkv.shape[0]
         heads = qkv[:, : (hq + hkv) * d].view(t, hq + hkv, d)
         x = heads.float()
@@ -200,7 +200,7 @@ class EmulatedOps:
         if norm_dim:
             x = x * torch.rsqrt((x * x).sum(-1, keepdim=True) / norm_dim + norm_eps)
         if q_weight is not None:
-            x[:, :hq] = x[:, :hq] * q_weight
+            x[:, :hq] = x[:, :hq] * (q_weight.view(hq, d) if q_weight_per_head else q_weight)
         if k_weight is not None:
             x[:, hq:] = x[:, hq:] * k_weight
         heads.copy_(x.to(qkv.dtype))
@@ -210,24 +210,119 @@ class EmulatedOps:
             vals = raw_keys if values_from_keys else qkv[:, (hq + hkv) * d:].view(t, hkv, d)
             kv[:, 1].view(kv.shape[0], hkv, d, PAGE)[page, :, :, off] = vals
 
-    def moe_route(self, x, w_router, chosen, weight, w_router_act=None) -> None:
-        s = torch.sigmoid(x.float() @ w_router.float().T)
+    def moe_route(self, x, w_router, chosen, weight, w_router_act=None, bias=None, mode=0) -> None:
+        z = x.float() @ w_router.float().T
+        if bias is not None:
+            z = z + bias
+        s = torch.sigmoid(z) if mode == 0 else z
         order = torch.argsort(-s, dim=-1, stable=True)[:, : chosen.shape[1]]
         chosen.copy_(order.to(torch.int32))
-        weight.copy_(torch.gather(s, 1, order))
+        picked = torch.gather(s, 1, order)
+        weight.copy_(picked if mode == 0 else torch.softmax(picked, dim=-1))
 
-    def moe_experts(self, x, chosen, weight, w_gate_up, w_down, act, out, gate_alpha, limit, up_shift) -> None:
+    def moe_experts(self, x, chosen, weight, w_gate_up, w_down, act, out, gate_alpha, limit, up_shift,
+                    weight_on_output=False) -> None:
         t, k = chosen.shape
         f = w_gate_up.shape[1] // 2
         for i in range(t):
             for j in range(k):
                 e = int(chosen[i, j])
-                h = x[i].float() * weight[i, j]
+                h = x[i].float() * (1.0 if weight_on_output else weight[i, j])
                 gu = w_gate_up[e].float() @ h
                 g, u = gu[:f].clamp(max=limit), gu[f:].clamp(-limit, limit)
                 y = (g * torch.sigmoid(gate_alpha * g) * (u + up_shift)).to(act.dtype)
                 act[i * k + j] = y
-                out[j, i] = w_down[e].float() @ y.float()
+                out[j, i] = (w_down[e].float() @ y.float()) * (weight[i, j] if weight_on_output else 1.0)
+
+    def row_gate(self, out, x, w) -> None:
+        out.mul_(torch.sigmoid(x.float() @ w)[:, None])
+
+    def layernorm_step(self, residual, delta, post, pre, out, rows=None) -> None:
+        def ln(y, terms):
+            w, b, eps = terms
+            d = y - y.mean(-1, keepdim=True)
+            return d * torch.rsqrt((d * d).mean(-1, keepdim=True) + eps) * w + b
+
+        if delta is not None:
+            residual.add_(ln(delta.float().sum(0) if delta.dim() == 3 else delta.float(), post))
+        if out is not None:
+            out.copy_(ln(residual if rows is None else residual[rows.long()], pre).to(out.dtype))
+
+    def add_sinusoid(self, x, positions, freq) -> None:
+        h = x.shape[1]
+        ang = positions.double()[:, None] * freq[torch.arange(h) // 2][None, :]
+        x.add_(torch.where(torch.arange(h) % 2 == 0, torch.sin(ang), torch.cos(ang)).float())
+
+    def short_conv(self, rows, col, conv_w, out, state, state_offset, ctx, silu=True) -> None:
+        channels, taps = conv_w.shape
+        keep = taps - 1
+        starts = ctx.item_start.tolist()
+        for i in range(ctx.num_items):
+            t0, t1 = starts[i], starts[i + 1]
+            saved = state[int(ctx.slots[i]), state_offset: state_offset + keep * channels].view(keep, channels)
+            v = torch.cat([saved, rows[t0:t1, col: col + channels].float()], dim=0)
+            acc = torch.zeros((t1 - t0, channels))
+            for j in range(taps):
+                acc += conv_w[:, j] * v[j: j + t1 - t0]
+            out[t0:t1] = torch.nn.functional.silu(acc) if silu else acc
+            if keep:
+                saved.copy_(v[-keep:].clone())
+
+    def gated_delta_prepare(self, u, groups, dim, gates, decay_log, decay_bias, coef, q_scale, unit_eps) -> None:
+        t, heads = u.shape[0], decay_log.numel()
+        qk = u[:, : 2 * groups * dim].view(t, 2 * groups, dim)
+        unit = qk * torch.rsqrt((qk * qk).sum(-1, keepdim=True) + unit_eps)
+        unit[:, :groups] *= q_scale
+        qk.copy_(unit)
+        b = torch.sigmoid(gates[:, :heads])
+        g = torch.exp(-torch.exp(decay_log) * torch.nn.functional.softplus(gates[:, heads:] + decay_bias))
+        coef.copy_(torch.cat([g, -b, b], dim=-1))
+
+    def general_delta_prepare(self, rows, r_col, k_col, v_col, a_col, l_col, rate_bias, decay_out, decay_bias, operands,
+                              heads, dim, decay_floor, unit_eps) -> None:
+        t, hd = rows.shape[0], heads * dim
+        r, k, v, a = (rows[:, c: c + hd].float() for c in (r_col, k_col, v_col, a_col))
+        low = torch.tanh(rows[:, l_col: l_col + decay_out.shape[1]].float()) @ decay_out.T + decay_bias
+        w = torch.exp(-decay_floor * torch.sigmoid(low))
+        kh = k.view(t, heads, dim)
+        c = (kh * torch.rsqrt((kh * kh).sum(-1, keepdim=True) + unit_eps)).reshape(t, hd)
+        operands.copy_(torch.cat([r, k, v, w, -torch.sigmoid(a + rate_bias) * c, c], dim=-1))
+
+    def delta_scan(self, keys, directions, removals, queries, key_groups, decay_vectors, decay, removal_scale,
+                   value_scale, values, out, state, state_offset, ctx, heads, dim, vdim, reads_decayed) -> None:
+        t = out.shape[0]
+
+        def vec(pair, n, size):
+            return pair[0][:, pair[1]: pair[1] + n * size].view(t, n, size)
+
+        def num(pair):
+            return torch.ones((t, heads)) if pair is None else pair[0][:, pair[1]: pair[1] + heads]
+
+        rep = heads // key_groups
+        kk, cc, pp, rr = (vec(p, key_groups, dim).repeat_interleave(rep, dim=1) for p in (keys, directions, removals, queries))
+        dv = torch.ones((t, heads, dim)) if decay_vectors is None else vec(decay_vectors, heads, dim)
+        ds, ps, xs = num(decay), num(removal_scale), num(value_scale)
+        xx = vec(values, heads, vdim)
+        o = out.view(t, heads, vdim)
+        starts = ctx.item_start.tolist()
+        for i in range(ctx.num_items):
+            st = state[int(ctx.slots[i]), state_offset: state_offset + heads * vdim * dim].view(heads, vdim, dim)
+            s = st.clone().transpose(1, 2)                                   # [heads, dim, vdim]
+            for k in range(starts[i], starts[i + 1]):
+                dec = (dv[k] * ds[k][:, None])[:, :, None] * s
+                dot = torch.einsum("hd,hdv->hv", cc[k], dec if reads_decayed else s)
+                s = dec + (ps[k][:, None] * pp[k])[:, :, None] * dot[:, None, :] \
+                    + kk[k][:, :, None] * (xs[k][:, None] * xx[k])[:, None, :]
+                o[k] = torch.einsum("hd,hdv->hv", rr[k], s)
+            st.copy_(s.transpose(1, 2))
+
+    def heads_norm_gate(self, o, heads, vdim, weight, weight_per_head, eps, gate_rows, gate_col, activation, out) -> None:
+        t = o.shape[0]
+        y = o.view(t, heads, vdim)
+        y = y * torch.rsqrt((y * y).mean(-1, keepdim=True) + eps) * (weight.view(heads, vdim) if weight_per_head else weight)
+        z = gate_rows[:, gate_col: gate_col + heads * vdim].float().view(t, heads, vdim)
+        act = torch.nn.functional.silu(z) if activation == "silu" else torch.sigmoid(z)
+        out.copy_((y * act).reshape(t, heads * vdim).to(out.dtype))
 
     def expand_kv(self, x, rep):
         """[keys, kv_heads, d] -> [keys, heads, d]: query head h reads kv head h // rep."""
