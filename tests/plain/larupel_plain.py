@@ -266,3 +266,13 @@ class PlainLarupel:
             streams.append(x)
         logits = self.norm(x, "final.norm") @ self.w["head"].T
         return (logits, np.stack(streams)) if return_layers else logits
+
+    def logits(self, tokens) -> np.ndarray:
+        return self.forward(tokens)
+
+    def greedy(self, prompt, n: int) -> list[int]:
+        """The n tokens greedy decoding makes behind ``prompt`` (the whole sequence is run again for each)."""
+        seq = list(prompt)
+        for _ in range(n):
+            seq.append(int(np.argmax(self.forward(seq)[-1])))
+        return seq[len(prompt):]
