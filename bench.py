@@ -124,8 +124,41 @@ def gokolix_pair(size: dict, layers: int, vocab: int) -> tuple[dict, dict]:
     return gokolix, llama
 
 
+# Larupel at sizes that resemble real layers, beside the Llama decoder of equal size: same width, the
+# attention layers' head counts and head size, and an inner feed-forward size that a token passes
+# through in both (dense: ff; experts: top x ff plus the shared expert). Four layers: a gated delta rule
+# behind convolutions with a dense feed-forward, a generalized delta rule, attention, and attention that
+# reads the layer before it, the last three with experts beside a shared one.
+LARUPEL_SIZES = {
+    "larupel-w2048-h32x64-ff8192": dict(width=2048, heads=32, kv_heads=8, dim=64, ff=8192, delta_heads=16, delta_kv=8, delta_dim=128,
+                                        general_heads=32, general_dim=64, rank=64, experts=32, expert_ff=1024, top=7),
+    "larupel-w4096-h32x128-ff14336": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=14336, delta_heads=32, delta_kv=16,
+                                          delta_dim=128, general_heads=64, general_dim=64, rank=128, experts=16, expert_ff=3584, top=3),
+}
+
+
+def larupel_pair(size: dict, layers: int, vocab: int) -> tuple[dict, dict]:
+    """(Larupel config.json, the Llama config.json of equal size). ``layers`` is not used: the pattern has four."""
+    experts = {"kind": "moe", "router": {"experts": size["experts"], "top": size["top"]}, "expert": {"ff": size["expert_ff"]},
+               "shared": {"ff": size["ff"] - size["top"] * size["expert_ff"]}}
+    att = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"], "scale": size["dim"] ** -0.5}
+    entries = [
+        {"type": "delta", "mlp": {"kind": "dense", "ff": size["ff"]},
+         "mixer": {"heads": size["delta_heads"], "kv_heads": size["delta_kv"], "dim": size["delta_dim"], "vdim": size["delta_dim"], "conv": 4}},
+        {"type": "general_delta", "mlp": experts,
+         "mixer": {"heads": size["general_heads"], "dim": size["general_dim"], "decay_rank": size["rank"]}},
+        {"type": "attention", "mlp": experts, "mixer": att},
+        {"type": "attention", "mlp": experts, "mixer": dict(att, kv_from=2)},
+    ]
+    larupel = {"architecture": "Larupel", "vocab": vocab, "width": size["width"], "norm": {"eps": 1e-5}, "layers": entries}
+    llama = dict(LLAMA_1B, vocab_size=vocab, hidden_size=size["width"], intermediate_size=size["ff"], num_hidden_layers=4,
+                 num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                 tie_word_embeddings=False)
+    return larupel, llama
+
+
 def compare_designs(args) -> int:
-    """Prefill and decode throughput of another design's layers (Radivik, Gokolix) beside Llama layers of
+    """Prefill and decode throughput of another design's layers (Radivik, Gokolix, Larupel) beside Llama layers of
     equal size, through the same runner and step function. One JSON line; the default benchmark is not run."""
     import numpy as np
     import torch
@@ -137,7 +170,10 @@ def compare_designs(args) -> int:
     rng = np.random.default_rng(0)
     vocab, layers = 32000, args.layers or 4
     prompt, batch, context = args.prompt_len, args.batch, args.context
-    if args.compare in GOKOLIX_SIZES or args.compare == "gokolix":
+    if args.compare in LARUPEL_SIZES or args.compare == "larupel":
+        design, pair_of = "larupel", larupel_pair
+        sizes = LARUPEL_SIZES if args.compare == "larupel" else {args.compare: LARUPEL_SIZES[args.compare]}
+    elif args.compare in GOKOLIX_SIZES or args.compare == "gokolix":
         design, pair_of = "gokolix", gokolix_pair
         sizes = GOKOLIX_SIZES if args.compare == "gokolix" else {args.compare: GOKOLIX_SIZES[args.compare]}
     else:
@@ -253,11 +289,12 @@ def main() -> int:
     ap.add_argument("--no-peaks", action="store_true", help="skip measuring the copy bandwidth and a large library product")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.2-1b", help="layer sizes of the random model")
-    ap.add_argument("--compare", choices=sorted(RADIVIK_SIZES) + ["all"] + sorted(GOKOLIX_SIZES) + ["gokolix"], default=None,
-                    help="instead of the benchmark: Radivik or Gokolix layers of this size ('all': every Radivik size, "
-                         "'gokolix': every Gokolix size) beside Llama layers of equal size (prefill of --prompt-len tokens, "
+    ap.add_argument("--compare", choices=sorted(RADIVIK_SIZES) + ["all"] + sorted(GOKOLIX_SIZES) + ["gokolix"] + sorted(LARUPEL_SIZES) + ["larupel"],
+                    default=None,
+                    help="instead of the benchmark: Radivik, Gokolix or Larupel layers of this size ('all': every Radivik size, "
+                         "'gokolix' / 'larupel': every size of that design) beside Llama layers of equal size (prefill of --prompt-len tokens, "
                          "decoding at --batch in --context; --layers, default 4, for Radivik)")
-    ap.add_argument("--compare-only", choices=["both", "radivik", "gokolix", "llama"], default="both")
+    ap.add_argument("--compare-only", choices=["both", "radivik", "gokolix", "larupel", "llama"], default="both")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

@@ -137,8 +137,9 @@ def route(logits: np.ndarray, top: int) -> tuple[np.ndarray, np.ndarray]:
     return order, z / z.sum(axis=-1, keepdims=True)
 
 
-def gated_ff(h: np.ndarray, gate: np.ndarray, up: np.ndarray, down: np.ndarray, act) -> np.ndarray:
-    return (act(h @ gate.T) * (h @ up.T)) @ down.T
+def gated_ff(h: np.ndarray, gate: np.ndarray, up: np.ndarray, down: np.ndarray, act, r=lambda x: x) -> np.ndarray:
+    """``r`` rounds what an engine would hold in its activation type: the gated product."""
+    return r(act(h @ gate.T) * (h @ up.T)) @ down.T
 
 
 # ---------------------------------------------------------------------- model
@@ -147,20 +148,30 @@ def gated_ff(h: np.ndarray, gate: np.ndarray, up: np.ndarray, down: np.ndarray, 
 class PlainLarupel:
     """``weights``: name -> float64 array (as the checkpoint names them); ``cfg``: config.json as a dict."""
 
-    def __init__(self, cfg: dict[str, Any], weights: dict[str, np.ndarray]) -> None:
+    def __init__(self, cfg: dict[str, Any], weights: dict[str, np.ndarray], bf16: bool = False) -> None:
+        """``bf16``: the yardstick for a 16-bit engine. The outputs of the norms, of the products with
+        weight matrices and of the activations behind them, queries and keys as attention uses them, and
+        every sub-layer's output are rounded to bfloat16; everything the recurrences take in behind their
+        projections, scores, softmaxes, router logits and the stream are not. How far that moves the logits
+        of a model is what an engine that computes in bfloat16 may be off by, whatever its order of sums."""
+        self.r = (lambda x: round_bf16(np.asarray(x, dtype=np.float32)).astype(np.float64)) if bf16 else (lambda x: x)
         self.cfg = cfg
         self.w = {k: np.asarray(v, dtype=np.float64) for k, v in weights.items()}
         self.eps = float(cfg["norm"]["eps"])
         self.width = int(cfg["width"])
 
     @classmethod
-    def from_dir(cls, model_dir: str | Path) -> "PlainLarupel":
+    def from_dir(cls, model_dir: str | Path, bf16: bool = False) -> "PlainLarupel":
         model_dir = Path(model_dir)
         cfg = json.loads((model_dir / "config.json").read_text())
-        return cls(cfg, read_safetensors(model_dir / "model.safetensors"))
+        return cls(cfg, read_safetensors(model_dir / "model.safetensors"), bf16)
 
     def norm(self, x: np.ndarray, name: str) -> np.ndarray:
         return layer_norm(x, self.w[name], self.w[name + ".b"], self.eps)
+
+    def lin(self, h: np.ndarray, name: str) -> np.ndarray:
+        """h W^T, as an engine's activation type holds it."""
+        return self.r(h @ self.w[name].T)
 
     # ----- mixers
 
@@ -168,9 +179,9 @@ class PlainLarupel:
         w = self.w
         heads, groups, dim, vdim = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
         n = h.shape[0]
-        q = silu(short_conv(h @ w[p + "q"].T, w[p + "q.conv"])).reshape(n, groups, dim)
-        k = silu(short_conv(h @ w[p + "k"].T, w[p + "k.conv"])).reshape(n, groups, dim)
-        v = silu(short_conv(h @ w[p + "v"].T, w[p + "v.conv"])).reshape(n, heads, vdim)
+        q = silu(short_conv(self.lin(h, p + "q"), w[p + "q.conv"])).reshape(n, groups, dim)
+        k = silu(short_conv(self.lin(h, p + "k"), w[p + "k.conv"])).reshape(n, groups, dim)
+        v = silu(short_conv(self.lin(h, p + "v"), w[p + "v.conv"])).reshape(n, heads, vdim)
         q = unit_length(q) * dim ** -0.5
         k = unit_length(k)
         strength = sigmoid(h @ w[p + "b"].T)                                                    # [n, heads]
@@ -180,62 +191,62 @@ class PlainLarupel:
             g = hd // (heads // groups)
             out[:, hd] = gated_delta(q[:, g], k[:, g], v[:, hd], strength[:, hd], decay[:, hd])
         out = unit_rms(out, self.eps) * w[p + "norm"][None, None, :]
-        out = out.reshape(n, heads * vdim) * silu(h @ w[p + "g"].T)
-        return out @ w[p + "o"].T
+        out = self.r(out.reshape(n, heads * vdim) * silu(self.lin(h, p + "g")))
+        return self.lin(out, p + "o")
 
     def mix_general_delta(self, h: np.ndarray, p: str, m: dict[str, Any]) -> np.ndarray:
         w = self.w
         heads, dim = int(m["heads"]), int(m["dim"])
         n = h.shape[0]
-        r = (h @ w[p + "r"].T).reshape(n, heads, dim)
-        k = (h @ w[p + "k"].T).reshape(n, heads, dim)
-        v = (h @ w[p + "v"].T).reshape(n, heads, dim)
-        low = np.tanh(h @ w[p + "w1"].T) @ w[p + "w2"].T + w[p + "w0"][None, :]
+        r = self.lin(h, p + "r").reshape(n, heads, dim)
+        k = self.lin(h, p + "k").reshape(n, heads, dim)
+        v = self.lin(h, p + "v").reshape(n, heads, dim)
+        low = np.tanh(self.lin(h, p + "w1")) @ w[p + "w2"].T + w[p + "w0"][None, :]
         decay = np.exp(-DECAY_FLOOR * sigmoid(low)).reshape(n, heads, dim)
-        rate = sigmoid(h @ w[p + "a"].T + w[p + "a.b"][None, :]).reshape(n, heads, dim)
+        rate = sigmoid(self.lin(h, p + "a") + w[p + "a.b"][None, :]).reshape(n, heads, dim)
         out = np.zeros((n, heads, dim))
         for hd in range(heads):
             out[:, hd] = generalized_delta(r[:, hd], k[:, hd], v[:, hd], decay[:, hd], rate[:, hd])
         out = unit_rms(out, self.eps).reshape(n, heads * dim) * w[p + "norm"][None, :]
-        out = out * sigmoid(h @ w[p + "g"].T)
-        return out @ w[p + "o"].T
+        out = self.r(out * sigmoid(self.lin(h, p + "g")))
+        return self.lin(out, p + "o")
 
     def keys_values(self, h: np.ndarray, p: str, m: dict[str, Any]) -> tuple[np.ndarray, np.ndarray]:
         w = self.w
         groups, dim, vdim = int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
         n = h.shape[0]
-        k = unit_rms((h @ w[p + "k"].T).reshape(n, groups, dim), self.eps) * w[p + "k.norm"][None, None, :]
-        v = (h @ w[p + "v"].T).reshape(n, groups, vdim)
-        return k, v
+        k = unit_rms(self.lin(h, p + "k").reshape(n, groups, dim), self.eps) * w[p + "k.norm"][None, None, :]
+        v = self.lin(h, p + "v").reshape(n, groups, vdim)
+        return self.r(k), v
 
     def mix_attention(self, h: np.ndarray, p: str, m: dict[str, Any], kv: tuple[np.ndarray, np.ndarray]) -> np.ndarray:
         w = self.w
         heads, groups, dim, vdim = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
         n = h.shape[0]
-        q = unit_rms((h @ w[p + "q"].T).reshape(n, heads, dim), self.eps) * w[p + "q.norm"][None, None, :]
+        q = self.r(unit_rms(self.lin(h, p + "q").reshape(n, heads, dim), self.eps) * w[p + "q.norm"][None, None, :])
         k, v = kv
         out = np.zeros((n, heads, vdim))
         for hd in range(heads):
             g = hd // (heads // groups)
             out[:, hd], _ = causal_softmax_attention(q[:, hd], k[:, g], v[:, g], float(m["scale"]) * w[p + "temp"][hd])
-        return out.reshape(n, heads * vdim) @ w[p + "o"].T
+        return self.lin(self.r(out.reshape(n, heads * vdim)), p + "o")
 
     # ----- feed-forwards
 
     def feed_forward(self, h: np.ndarray, p: str, f: dict[str, Any]) -> np.ndarray:
         w = self.w
         if f["kind"] == "dense":
-            return gated_ff(h, w[p + "gate"], w[p + "up"], w[p + "down"], gelu_tanh)
+            return self.r(gated_ff(h, w[p + "gate"], w[p + "up"], w[p + "down"], gelu_tanh, self.r))
         top = int(f["router"]["top"])
         chosen, weight = route(h @ w[p + "router"].T + w[p + "router.b"][None, :], top)
         out = np.zeros_like(h)
         for t in range(h.shape[0]):
             for e, wt in zip(chosen[t], weight[t]):
                 q = f"{p}e{e}."
-                out[t] += wt * gated_ff(h[t: t + 1], w[q + "gate"], w[q + "up"], w[q + "down"], silu)[0]
+                out[t] += wt * gated_ff(h[t: t + 1], w[q + "gate"], w[q + "up"], w[q + "down"], silu, self.r)[0]
         if f.get("shared") is not None:
             q = p + "shared."
-            out += gated_ff(h, w[q + "gate"], w[q + "up"], w[q + "down"], silu) * sigmoid(h @ w[q + "sg"].T)
+            out += gated_ff(h, w[q + "gate"], w[q + "up"], w[q + "down"], silu, self.r) * sigmoid(h @ w[q + "sg"].T)
         return out
 
     # ----- the model
@@ -249,7 +260,7 @@ class PlainLarupel:
         streams = []
         for i, layer in enumerate(self.cfg["layers"]):
             p, m = f"l{i}.", layer["mixer"]
-            h = self.norm(x, p + "norm1")
+            h = self.r(self.norm(x, p + "norm1"))
             if layer["type"] == "delta":
                 y = self.mix_delta(h, p + "mix.", m)
             elif layer["type"] == "general_delta":
@@ -262,9 +273,9 @@ class PlainLarupel:
                 raise ValueError(layer["type"])
             x = x + self.norm(y, p + "norm1b")
             if layer.get("mlp") is not None:
-                x = x + self.norm(self.feed_forward(self.norm(x, p + "norm2"), p + "mlp.", layer["mlp"]), p + "norm2b")
+                x = x + self.norm(self.feed_forward(self.r(self.norm(x, p + "norm2")), p + "mlp.", layer["mlp"]), p + "norm2b")
             streams.append(x)
-        logits = self.norm(x, "final.norm") @ self.w["head"].T
+        logits = self.r(self.norm(x, "final.norm")) @ self.w["head"].T
         return (logits, np.stack(streams)) if return_layers else logits
 
     def logits(self, tokens) -> np.ndarray:
