@@ -30,6 +30,9 @@ namespace psamd {
 constexpr int kConvMaxTaps = 16;
 constexpr int kLPC = 16;      // lanes per column of the state
 constexpr int kCols = 16;     // columns per workgroup
+// Tokens whose vectors are in LDS at a time: 40 KB of vectors at most, and no more runs' worth of
+// registers per thread than eight entries of each vector.
+template <int E> constexpr int kScanRun = E == 16 ? 8 : 16;
 
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
 __device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
@@ -114,51 +117,81 @@ __global__ __launch_bounds__(256) void gated_delta_prepare_kernel(
 
 // ------------------------------------------------------------------ operands of the generalized delta rule
 
-// grid (tokens, heads), 256 threads over the head's channels. rows (activation type) hold r, k, v,
+// grid (ceil(tokens / 4), heads), 256 threads: four tokens of one head, so that a row of the low-rank
+// map's outer matrix is fetched once for four tokens. rows (activation type) hold r, k, v,
 // the removal rate's logits (heads x dim each, at their columns) and the low-rank map's inner
 // values (rank, at l_col). ops row = [r | k | v | w | p | c], heads x dim each, float:
-//   w = exp(-decay_floor * sigmoid(sum_j w2[hc, j] tanh(l[j]) + w0[hc])), c = k / sqrt(sum k^2 + unit_eps),
-//   p = -sigmoid(a + a_bias[hc]) * c.
+//   w = exp(-decay_floor * sigmoid(sum_j w2[j, hc] tanh(l[j]) + w0[hc])), c = k / sqrt(sum k^2 + unit_eps),
+//   p = -sigmoid(a + a_bias[hc]) * c. w2 is stored [rank][heads * dim].
+constexpr int kPrepTokens = 4;
+
 template <typename A>
 __global__ __launch_bounds__(256) void general_delta_prepare_kernel(
     const A* __restrict__ rows, int64_t in_row, int r_col, int k_col, int v_col, int a_col, int l_col,
     const float* __restrict__ a_bias, const float* __restrict__ w2, const float* __restrict__ w0, float* __restrict__ ops,
-    int heads, int dim, int rank, float decay_floor, float unit_eps) {
-  extern __shared__ float prep_smem[];                 // tanh(l)[rank], then 4 floats for the sum
-  const int64_t t = blockIdx.x;
+    int64_t tokens, int heads, int dim, int rank, float decay_floor, float unit_eps) {
+  extern __shared__ float prep_smem[];                 // tanh(l)[4][rank], then 1 / |k| of the four tokens
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kPrepTokens;
+  const int nt = static_cast<int>(min(static_cast<int64_t>(kPrepTokens), tokens - t0));
   const int h = blockIdx.y;
-  const A* row = rows + t * in_row;
-  for (int j = threadIdx.x; j < rank; j += blockDim.x) prep_smem[j] = tanhf(to_float<A>(row[l_col + j]));
-  float ss = 0.f;
-  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
-    const float k = to_float<A>(row[k_col + h * dim + i]);
-    ss = fmaf(k, k, ss);
+  float* inv = prep_smem + kPrepTokens * rank;
+  for (int idx = threadIdx.x; idx < nt * rank; idx += blockDim.x) {
+    const int tk = idx / rank, j = idx - tk * rank;
+    prep_smem[idx] = tanhf(to_float<A>(rows[(t0 + tk) * in_row + l_col + j]));
   }
-  ss = block_sum(ss, prep_smem + rank, 4);             // its barriers also publish the tanh values
-  const float inv = 1.f / sqrtf(ss + unit_eps);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  if (wave < nt) {
+    const A* row = rows + (t0 + wave) * in_row + k_col + static_cast<int64_t>(h) * dim;
+    float ss = 0.f;
+    for (int i = lane; i < dim; i += kWave) {
+      const float k = to_float<A>(row[i]);
+      ss = fmaf(k, k, ss);
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) inv[wave] = 1.f / sqrtf(ss + unit_eps);
+  }
+  __syncthreads();
   const int64_t hd = static_cast<int64_t>(heads) * dim;
-  float* o = ops + t * 6 * hd + static_cast<int64_t>(h) * dim;
-  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+  for (int idx = threadIdx.x; idx < nt * dim; idx += blockDim.x) {
+    const int tk = idx / dim, i = idx - tk * dim;
+    const A* row = rows + (t0 + tk) * in_row;
     const int64_t hc = static_cast<int64_t>(h) * dim + i;
-    const float* w2r = w2 + hc * rank;
+    const float* w2c = w2 + hc;                          // column hc of the map stored [rank][heads * dim]: lanes read side by side
+    const float* th = prep_smem + tk * rank;
     float low = w0[hc];
-    for (int j = 0; j < rank; ++j) low = fmaf(w2r[j], prep_smem[j], low);
+    for (int j = 0; j < rank; ++j) low = fmaf(w2c[j * hd], th[j], low);
     const float k = to_float<A>(row[k_col + hc]);
-    const float c = k * inv;
-    o[i] = to_float<A>(row[r_col + hc]);
-    o[hd + i] = k;
-    o[2 * hd + i] = to_float<A>(row[v_col + hc]);
-    o[3 * hd + i] = expf(-decay_floor * sigmoidf_(low));
-    o[4 * hd + i] = -sigmoidf_(to_float<A>(row[a_col + hc]) + a_bias[hc]) * c;
-    o[5 * hd + i] = c;
+    const float c = k * inv[tk];
+    float* o = ops + (t0 + tk) * 6 * hd + hc;
+    o[0] = to_float<A>(row[r_col + hc]);
+    o[hd] = k;
+    o[2 * hd] = to_float<A>(row[v_col + hc]);
+    o[3 * hd] = expf(-decay_floor * sigmoidf_(low));
+    o[4 * hd] = -sigmoidf_(to_float<A>(row[a_col + hc]) + a_bias[hc]) * c;
+    o[5 * hd] = c;
   }
 }
 
 // ------------------------------------------------------------------ the recurrence
 
+// Sum over the 16 lanes of a row, in every lane, by four data-parallel moves inside the vector unit (lane
+// pairs, pairs of pairs, the mirrored half row, the mirrored row) instead of four trips through LDS: the
+// recurrence waits on this sum once per token.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+  return v;
+}
+
 // grid (items, heads, ceil(vdim / 16)), 256 threads: column col = threadIdx.x / 16 of the block's 16,
 // lane l of its 16 holds the E entries l * E .. l * E + E - 1 of the column (dim <= 16 E). The vectors
-// of `tt` tokens at a time pass through LDS.
+// of TT tokens at a time pass through LDS; the run after is already on its way from memory, in
+// registers, while a run is walked. A token costs one dependent sum over the column: with
+// dec = d * S and take = ps (c . S*), the new column is dec + p take + k xw, and its read-out
+// r . S is (r . dec) + take (r . p) + xw (r . k), where r . dec is summed beside c . S* and the two
+// products of vectors alone are formed once per token for all columns when the run arrives.
 template <int E>
 __global__ __launch_bounds__(256) void delta_scan_kernel(
     const float* __restrict__ kvec, const float* __restrict__ cvec, const float* __restrict__ pvec,
@@ -166,12 +199,14 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
     const float* __restrict__ dscal, const float* __restrict__ pscal, const float* __restrict__ xscal, int64_t scal_row,
     const float* __restrict__ x, int64_t x_row, float* __restrict__ out, int64_t out_row, float* __restrict__ state,
     int64_t state_row, const int32_t* __restrict__ item_start, const int32_t* __restrict__ slots, int dim, int vdim,
-    int reads_decayed, int tt) {
+    int reads_decayed) {
   constexpr int DP = E * kLPC;                          // the column's length, padded
-  extern __shared__ __align__(16) float scan_smem[];   // [tt][5][DP] k, c, p, r, d; [tt][4] d, ps, xs; [tt][kCols] x
-  float* vec = scan_smem;
-  float* sca = vec + static_cast<int64_t>(tt) * 5 * DP;
-  float* xs_ = sca + tt * 4;
+  constexpr int TT = kScanRun<E>;                       // tokens per run
+  constexpr int VPT = TT * DP / 256;                    // vector entries a thread carries per run
+  constexpr int NS = 6;                                 // numbers per token: d, ps, xs, r . p, r . k
+  __shared__ __align__(16) float vec[TT * 5 * DP];      // [TT][5][DP] k, c, p, r, d
+  __shared__ float sca[TT * NS];
+  __shared__ float xs_[TT * kCols];
   const int item = blockIdx.x, h = blockIdx.y, g = h / heads_per_group;
   const int col = threadIdx.x / kLPC, l = threadIdx.x % kLPC;
   const int j0 = blockIdx.z * kCols, j = j0 + col;
@@ -180,53 +215,87 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   float s[E];
 #pragma unroll
   for (int e = 0; e < E; ++e) s[e] = (j < vdim && l * E + e < dim) ? st[e] : 0.f;
-  for (int64_t t0 = s0; t0 < s1; t0 += tt) {
-    const int n = static_cast<int>(min(static_cast<int64_t>(tt), s1 - t0));
-    __syncthreads();                                    // everybody is done with the run before
-    for (int idx = threadIdx.x; idx < n * DP; idx += 256) {
-      const int tk = idx / DP, i = idx % DP;
-      const int64_t at = (t0 + tk) * key_row + static_cast<int64_t>(g) * dim + i;
-      const bool in = i < dim;
-      float* v = vec + (static_cast<int64_t>(tk) * 5) * DP + i;
-      v[0] = in ? kvec[at] : 0.f;
-      v[DP] = in ? cvec[at] : 0.f;
-      v[2 * DP] = in ? pvec[at] : 0.f;
-      v[3 * DP] = in ? rvec[at] : 0.f;
-      v[4 * DP] = (in && dvec != nullptr) ? dvec[(t0 + tk) * dvec_row + static_cast<int64_t>(h) * dim + i] : 1.f;
+
+  float fk[VPT], fc[VPT], fp[VPT], fr[VPT], fd[VPT], fx = 0.f, fs = 1.f;
+  // Round tf fetches the run from token tf on into registers and walks the run before it, which the
+  // round before fetched: the loads are in flight while the tokens are walked.
+  for (int64_t tf = s0; tf < s1 + TT; tf += TT) {
+    const int64_t t0 = tf - TT;                         // the run that is walked
+    const int n = static_cast<int>(min(static_cast<int64_t>(TT), s1 - t0));
+    if (tf > s0) {
+      __syncthreads();                                  // everybody is done with the run before
+#pragma unroll
+      for (int u = 0; u < VPT; ++u) {
+        const int idx = threadIdx.x + u * 256, tk = idx / DP, i = idx % DP;
+        float* v = vec + tk * 5 * DP + i;
+        v[0] = fk[u];
+        v[DP] = fc[u];
+        v[2 * DP] = fp[u];
+        v[3 * DP] = fr[u];
+        v[4 * DP] = fd[u];
+      }
+      if (threadIdx.x / kCols < TT) xs_[threadIdx.x] = fx;
+      if (threadIdx.x < TT * 3) sca[(threadIdx.x / 3) * NS + threadIdx.x % 3] = fs;
+      __syncthreads();
     }
-    for (int idx = threadIdx.x; idx < n; idx += 256) {
-      const int64_t at = (t0 + idx) * scal_row + h;
-      sca[idx * 4] = dscal != nullptr ? dscal[at] : 1.f;
-      sca[idx * 4 + 1] = pscal != nullptr ? pscal[at] : 1.f;
-      sca[idx * 4 + 2] = xscal != nullptr ? xscal[at] : 1.f;
+    if (tf < s1) {
+      const int m = static_cast<int>(min(static_cast<int64_t>(TT), s1 - tf));
+#pragma unroll
+      for (int u = 0; u < VPT; ++u) {
+        const int idx = threadIdx.x + u * 256, tk = idx / DP, i = idx % DP;
+        const bool in = tk < m && i < dim;
+        const int64_t at = (tf + tk) * key_row + static_cast<int64_t>(g) * dim + i;
+        fk[u] = in ? kvec[at] : 0.f;
+        fc[u] = in ? cvec[at] : 0.f;
+        fp[u] = in ? pvec[at] : 0.f;
+        fr[u] = in ? rvec[at] : 0.f;
+        fd[u] = (in && dvec != nullptr) ? dvec[(tf + tk) * dvec_row + static_cast<int64_t>(h) * dim + i] : 1.f;
+      }
+      {
+        const int tk = threadIdx.x / kCols, cc = threadIdx.x % kCols;
+        fx = (tk < m && j0 + cc < vdim) ? x[(tf + tk) * x_row + static_cast<int64_t>(h) * vdim + j0 + cc] : 0.f;
+      }
+      if (threadIdx.x < TT * 3) {
+        const int tk = threadIdx.x / 3, which = threadIdx.x % 3;
+        const float* src = which == 0 ? dscal : which == 1 ? pscal : xscal;
+        fs = (tk < m && src != nullptr) ? src[(tf + tk) * scal_row + h] : 1.f;
+      }
     }
-    for (int idx = threadIdx.x; idx < n * kCols; idx += 256) {
-      const int tk = idx / kCols, cc = idx % kCols;
-      xs_[idx] = j0 + cc < vdim ? x[(t0 + tk) * x_row + static_cast<int64_t>(h) * vdim + j0 + cc] : 0.f;
+    if (tf == s0) continue;
+    if (col < n) {                                      // r . p and r . k of token col, once for all columns
+      const float* v = vec + col * 5 * DP + l * E;
+      float rp = 0.f, rk = 0.f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        rp = fmaf(v[3 * DP + e], v[2 * DP + e], rp);
+        rk = fmaf(v[3 * DP + e], v[e], rk);
+      }
+      rp = row16_sum(rp);
+      rk = row16_sum(rk);
+      if (l == 0) {
+        sca[col * NS + 3] = rp;
+        sca[col * NS + 4] = rk;
+      }
     }
     __syncthreads();
     for (int tk = 0; tk < n; ++tk) {
-      const float* v = vec + (static_cast<int64_t>(tk) * 5) * DP + l * E;
-      const float ds = sca[tk * 4], ps = sca[tk * 4 + 1], xw = sca[tk * 4 + 2] * xs_[tk * kCols + col];
+      const float* v = vec + tk * 5 * DP + l * E;
+      const float* sc = sca + tk * NS;
+      const float ds = sc[0], ps = sc[1], xw = sc[2] * xs_[tk * kCols + col];
       float dec[E];
-      float dot = 0.f;
+      float dot = 0.f, rd = 0.f;
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         dec[e] = v[4 * DP + e] * ds * s[e];
         dot = fmaf(v[DP + e], reads_decayed ? dec[e] : s[e], dot);
+        rd = fmaf(v[3 * DP + e], dec[e], rd);
       }
-#pragma unroll
-      for (int o = kLPC / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o, kWave);
+      dot = row16_sum(dot);
+      rd = row16_sum(rd);
       const float take = ps * dot;
-      float read = 0.f;
 #pragma unroll
-      for (int e = 0; e < E; ++e) {
-        s[e] = fmaf(v[e], xw, fmaf(v[2 * DP + e], take, dec[e]));
-        read = fmaf(v[3 * DP + e], s[e], read);
-      }
-#pragma unroll
-      for (int o = kLPC / 2; o > 0; o >>= 1) read += __shfl_xor(read, o, kWave);
-      if (l == 0 && j < vdim) out[(t0 + tk) * out_row + static_cast<int64_t>(h) * vdim + j] = read;
+      for (int e = 0; e < E; ++e) s[e] = fmaf(v[e], xw, fmaf(v[2 * DP + e], take, dec[e]));
+      if (l == 0 && j < vdim) out[(t0 + tk) * out_row + static_cast<int64_t>(h) * vdim + j] = fmaf(xw, sc[4], fmaf(take, sc[3], rd));
     }
   }
 #pragma unroll
@@ -263,14 +332,14 @@ __global__ __launch_bounds__(256) void heads_norm_gate_kernel(const float* __res
 }
 
 template <int E>
-static int launch_delta_scan(hipStream_t s, dim3 grid, size_t smem, const float* kvec, const float* cvec, const float* pvec,
+static int launch_delta_scan(hipStream_t s, dim3 grid, const float* kvec, const float* cvec, const float* pvec,
                              const float* rvec, int64_t key_row, int heads_per_group, const float* dvec, int64_t dvec_row,
                              const float* dscal, const float* pscal, const float* xscal, int64_t scal_row, const float* x,
                              int64_t x_row, float* out, int64_t out_row, float* state, int64_t state_row,
-                             const int32_t* item_start, const int32_t* slots, int dim, int vdim, int reads_decayed, int tt) {
-  delta_scan_kernel<E><<<grid, dim3(256), smem, s>>>(kvec, cvec, pvec, rvec, key_row, heads_per_group, dvec, dvec_row, dscal,
+                             const int32_t* item_start, const int32_t* slots, int dim, int vdim, int reads_decayed) {
+  delta_scan_kernel<E><<<grid, dim3(256), 0, s>>>(kvec, cvec, pvec, rvec, key_row, heads_per_group, dvec, dvec_row, dscal,
                                                      pscal, xscal, scal_row, x, x_row, out, out_row, state, state_row,
-                                                     item_start, slots, dim, vdim, reads_decayed, tt);
+                                                     item_start, slots, dim, vdim, reads_decayed);
   return check_launch("psamd_delta_scan");
 }
 
@@ -319,23 +388,23 @@ int psamd_general_delta_prepare(void* stream, const void* rows, int act_dtype, i
                                 int v_col, int a_col, int l_col, const float* a_bias, const float* w2, const float* w0,
                                 float* ops, int64_t tokens, int heads, int dim, int rank, float decay_floor, float unit_eps) {
   PSAMD_REQUIRE(tokens >= 0 && heads > 0 && dim > 0 && rank > 0, "bad sizes");
-  PSAMD_REQUIRE(tokens <= 2147483647LL && heads <= 65535 && rank <= 8192, "too large for one launch");
+  PSAMD_REQUIRE(tokens <= 2147483647LL && heads <= 65535 && rank <= 3072, "too large for one launch (rank at most 3,072)");
   const int64_t hd = static_cast<int64_t>(heads) * dim;
   PSAMD_REQUIRE(std::max(std::max(r_col, k_col), std::max(v_col, a_col)) + hd <= in_row && l_col + rank <= in_row &&
                     std::min(std::min(std::min(r_col, k_col), std::min(v_col, a_col)), l_col) >= 0,
                 "columns outside the rows");
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>(tokens), static_cast<unsigned>(heads));
-  const size_t smem = sizeof(float) * (static_cast<size_t>(rank) + 4);
+  const dim3 grid(static_cast<unsigned>(ceil_div(tokens, kPrepTokens)), static_cast<unsigned>(heads));
+  const size_t smem = sizeof(float) * kPrepTokens * (static_cast<size_t>(rank) + 1);
   if (act_dtype == kBF16) {
     general_delta_prepare_kernel<bf16_t><<<grid, dim3(256), smem, s>>>(static_cast<const bf16_t*>(rows), in_row, r_col, k_col,
-                                                                      v_col, a_col, l_col, a_bias, w2, w0, ops, heads, dim,
-                                                                      rank, decay_floor, unit_eps);
+                                                                      v_col, a_col, l_col, a_bias, w2, w0, ops, tokens, heads,
+                                                                      dim, rank, decay_floor, unit_eps);
   } else if (act_dtype == kF32) {
     general_delta_prepare_kernel<float><<<grid, dim3(256), smem, s>>>(static_cast<const float*>(rows), in_row, r_col, k_col,
-                                                                     v_col, a_col, l_col, a_bias, w2, w0, ops, heads, dim, rank,
-                                                                     decay_floor, unit_eps);
+                                                                     v_col, a_col, l_col, a_bias, w2, w0, ops, tokens, heads, dim,
+                                                                     rank, decay_floor, unit_eps);
   } else {
     return fail("psamd_general_delta_prepare: activation dtype must be float32 or bfloat16");
   }
@@ -356,16 +425,12 @@ int psamd_delta_scan(void* stream, const float* kvec, const float* cvec, const f
   hipStream_t s = static_cast<hipStream_t>(stream);
   int e = 1;
   while (e * kLPC < dim) e *= 2;
-  const int dp = e * kLPC;
-  const size_t per_token = sizeof(float) * (5 * static_cast<size_t>(dp) + 4 + kCols);
-  const int tt = static_cast<int>(std::max<size_t>(1, std::min<size_t>(16, (48 * 1024) / per_token)));
-  const size_t smem = per_token * tt;
   const dim3 grid(static_cast<unsigned>(items), static_cast<unsigned>(heads), static_cast<unsigned>(ceil_div(vdim, kCols)));
   const int hpg = heads / key_groups;
 #define PSAMD_SCAN(E)                                                                                                  \
-  return launch_delta_scan<E>(s, grid, smem, kvec, cvec, pvec, rvec, key_row, hpg, dvec, dvec_row, dscal, pscal, xscal,  \
+  return launch_delta_scan<E>(s, grid, kvec, cvec, pvec, rvec, key_row, hpg, dvec, dvec_row, dscal, pscal, xscal,  \
                               scal_row, x, x_row, out, out_row, state, state_row, item_start, slots, dim, vdim,        \
-                              reads_decayed, tt)
+                              reads_decayed)
   switch (e) {
     case 1: PSAMD_SCAN(1);
     case 2: PSAMD_SCAN(2);

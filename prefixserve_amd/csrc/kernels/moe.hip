@@ -488,18 +488,17 @@ static int launch_experts_rows(hipStream_t s, const void* x, const int32_t* chos
 }
 
 // out[t, :] *= sigmoid(x[t] . w): one number per token on the output of a branch every token takes.
-// One wave per token, the dot product in float.
+// One workgroup per token, the dot product in float.
 template <typename A>
 __global__ __launch_bounds__(256) void row_gate_kernel(float* __restrict__ out, const A* __restrict__ x,
-                                                       const float* __restrict__ w, int64_t tokens, int out_hidden, int hidden) {
-  const int lane = threadIdx.x & (kWave - 1);
-  const int64_t t = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-  if (t >= tokens) return;
+                                                       const float* __restrict__ w, int out_hidden, int hidden) {
+  __shared__ float parts[4];
+  const int64_t t = blockIdx.x;
   float acc = 0.f;
-  for (int i = lane; i < hidden; i += kWave) acc = fmaf(to_float<A>(x[t * hidden + i]), w[i], acc);
-  const float g = 1.f / (1.f + expf(-wave_sum(acc)));
+  for (int i = threadIdx.x; i < hidden; i += 256) acc = fmaf(to_float<A>(x[t * hidden + i]), w[i], acc);
+  const float g = 1.f / (1.f + expf(-block_sum(acc, parts, 4)));
   float* o = out + t * out_hidden;
-  for (int i = lane; i < out_hidden; i += kWave) o[i] *= g;
+  for (int i = threadIdx.x; i < out_hidden; i += 256) o[i] *= g;
 }
 
 }  // namespace psamd
@@ -624,14 +623,14 @@ int psamd_moe_experts_grouped(void* stream, const void* x, const int32_t* chosen
 
 int psamd_row_gate(void* stream, float* out, const void* x, int act_dtype, const float* w, int64_t tokens, int out_hidden,
                    int hidden) {
-  PSAMD_REQUIRE(tokens >= 0 && out_hidden > 0 && hidden > 0 && ceil_div(tokens, 4) <= 2147483647LL, "bad sizes");
+  PSAMD_REQUIRE(tokens >= 0 && out_hidden > 0 && hidden > 0 && tokens <= 2147483647LL, "bad sizes");
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>(ceil_div(tokens, 4)));
+  const dim3 grid(static_cast<unsigned>(tokens));
   if (act_dtype == kBF16) {
-    row_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(out, static_cast<const bf16_t*>(x), w, tokens, out_hidden, hidden);
+    row_gate_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(out, static_cast<const bf16_t*>(x), w, out_hidden, hidden);
   } else if (act_dtype == kF32) {
-    row_gate_kernel<float><<<grid, dim3(256), 0, s>>>(out, static_cast<const float*>(x), w, tokens, out_hidden, hidden);
+    row_gate_kernel<float><<<grid, dim3(256), 0, s>>>(out, static_cast<const float*>(x), w, out_hidden, hidden);
   } else {
     return fail("psamd_row_gate: activation dtype must be float32 or bfloat16");
   }

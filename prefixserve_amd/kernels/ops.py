@@ -824,16 +824,16 @@ class HipOps:
                               decay_bias, operands, heads: int, dim: int, decay_floor: float, unit_eps: float) -> None:
         """From rows (a kernel dtype; r, k, v and the rate's logits [heads, dim] at their columns, the decay
         map's inner values [rank] at l_col) to operands float32 [T, 6 heads dim] = [r | k | v | w | p | c]:
-        w = exp(-decay_floor sigmoid(decay_out tanh(l) + decay_bias)), c = k / sqrt(sum k^2 + unit_eps) per head,
+        w = exp(-decay_floor sigmoid(tanh(l) decay_out + decay_bias)) with decay_out float32 [rank, heads dim], c = k / sqrt(sum k^2 + unit_eps) per head,
         p = -sigmoid(rate logits + rate_bias) * c."""
         t = rows.shape[0]
         hd = heads * dim
-        rank = decay_out.shape[1]
+        rank = decay_out.shape[0]
         self._need(rows.is_contiguous() and max(r_col, k_col, v_col, a_col) + hd <= rows.shape[1] and l_col + rank <= rows.shape[1]
                    and min(r_col, k_col, v_col, a_col, l_col) >= 0, "general_delta_prepare: columns outside the rows")
         self._need(operands.dtype == torch.float32 and operands.shape == (t, 6 * hd) and operands.is_contiguous(),
                    "general_delta_prepare: operands are float32 [T, 6 heads dim]")
-        for v, shape in ((rate_bias, (hd,)), (decay_out, (hd, rank)), (decay_bias, (hd,))):
+        for v, shape in ((rate_bias, (hd,)), (decay_out, (rank, hd)), (decay_bias, (hd,))):
             self._need(v.dtype == torch.float32 and tuple(v.shape) == shape and v.is_contiguous(), "general_delta_prepare: float32 parameters")
         self._ok(self.lib.psamd_general_delta_prepare(self._stream(), rows.data_ptr(), _code(rows.dtype), rows.shape[1], r_col, k_col,
                                                       v_col, a_col, l_col, rate_bias.data_ptr(), decay_out.data_ptr(),

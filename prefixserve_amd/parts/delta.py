@@ -159,7 +159,8 @@ class GeneralizedDeltaRule(Mixer):
         # [r | k | v | gate | rate logits | the decay map's inner values] from one product.
         self.w_in = rt.ops.prepare_matrix(torch.cat([tensors[n[key]] for key in ("r", "k", "v", "gate", "rate", "decay_in")], dim=0), rt)
         self.w_o = rt.ops.prepare_matrix(tensors[n["o"]], rt)
-        self.rate_bias, self.decay_out, self.decay_bias, self.norm_w = f32("rate_bias"), f32("decay_out"), f32("decay_bias"), f32("norm")
+        self.rate_bias, self.decay_bias, self.norm_w = f32("rate_bias"), f32("decay_bias"), f32("norm")
+        self.decay_out = f32("decay_out").t().contiguous()       # [rank, heads dim]: a kernel's lanes read channels side by side
 
     def weight_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_o, self.decay_out))

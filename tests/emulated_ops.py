@@ -282,7 +282,7 @@ class EmulatedOps:
                               heads, dim, decay_floor, unit_eps) -> None:
         t, hd = rows.shape[0], heads * dim
         r, k, v, a = (rows[:, c: c + hd].float() for c in (r_col, k_col, v_col, a_col))
-        low = torch.tanh(rows[:, l_col: l_col + decay_out.shape[1]].float()) @ decay_out.T + decay_bias
+        low = torch.tanh(rows[:, l_col: l_col + decay_out.shape[0]].float()) @ decay_out + decay_bias
         w = torch.exp(-decay_floor * torch.sigmoid(low))
         kh = k.view(t, heads, dim)
         c = (kh * torch.rsqrt((kh * kh).sum(-1, keepdim=True) + unit_eps)).reshape(t, hd)

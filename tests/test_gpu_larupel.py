@@ -29,10 +29,11 @@ DEV = "cuda:0"
 # cancels brings its rounding back to size one (4e-5 seen on the host), the median row is at 5e-7.
 F32_TOL = 1e-4
 # bfloat16, the same measure, against the plain model with its products and activations rounded to
-# bfloat16 (``bf16_bars``): the mean over a trace's rows, and how many rows lie far out. A single row may
-# be anywhere: in these tiny models a router's close call falls the other way after rounding, in the
-# yardstick as in the engine but not at the same token, and moves that row by tenths.
-BF16_MEAN_FACTOR, BF16_FAR_FACTOR, BF16_FAR_SHARE = 1.5, 2.0, 0.03
+# bfloat16 (``bf16_bars``): the median and the ninth decile of a trace's rows, and how many rows lie far
+# out. A single row may be anywhere: in these tiny models a router's close call falls the other way after
+# rounding, in the yardstick as in the engine but not at the same token, and moves that row (and, through
+# a state, some behind it) by tenths; a mean would follow those few rows.
+BF16_FACTOR, BF16_TAIL_FACTOR, BF16_FAR_FACTOR, BF16_FAR_SHARE = 1.5, 2.5, 2.0, 0.03
 
 
 @pytest.fixture(scope="module")
@@ -223,7 +224,7 @@ def test_generalized_delta_rule_continues_from_its_slot(ops, dtype, heads, dim, 
         rows = torch.cat([p for _, p in pieces]).contiguous()
         t = ctx.num_tokens
         operands = torch.empty(t, 6 * s_, device=DEV)
-        ops.general_delta_prepare(rows, 0, s_, 2 * s_, 4 * s_, 5 * s_, a_bias, w2, w0, operands, heads, dim, floor, 1e-6)
+        ops.general_delta_prepare(rows, 0, s_, 2 * s_, 4 * s_, 5 * s_, a_bias, w2.t().contiguous(), w0, operands, heads, dim, floor, 1e-6)
         o = torch.empty(t, s_, device=DEV)
         ops.delta_scan(keys=(operands, s_), directions=(operands, 5 * s_), removals=(operands, 4 * s_), queries=(operands, 0),
                        key_groups=heads, decay_vectors=(operands, 3 * s_), decay=None, removal_scale=None, value_scale=None,
@@ -296,22 +297,21 @@ LENGTHS = [70, 33, 97, 18, 64, 45, 1, 52, 2, 81, 29, 3]
 
 
 def bf16_bars(folder, truth, reqs, last=0):
-    """(mean, 99th percentile) of the rows (the ``last`` ones of each request, or all) of a plain bfloat16
-    run against the plain model in float64."""
+    """(median, ninth decile, 99th percentile) of the rows (the ``last`` ones of each request, or all) of a
+    plain bfloat16 run against the plain model in float64."""
     rough = plain.PlainLarupel.from_dir(folder, bf16=True)
     rows = np.concatenate([np.abs(rough.logits(t)[-last:] - w[-last:]).max(-1) / np.abs(w[-last:]).max(-1) for t, w in zip(reqs, truth)])
-    return float(rows.mean()), float(np.quantile(rows, 0.99))
+    return tuple(float(np.quantile(rows, q)) for q in (0.5, 0.9, 0.99))
 
 
 def check_rows(errors, dtype, bars=None):
     if dtype == "float32":
         assert max(errors) < F32_TOL, max(errors)
     else:
-        mean_bar, far_bar = bars
         e = np.asarray(errors)
-        far = float((e > BF16_FAR_FACTOR * far_bar).mean())
-        assert np.isfinite(e).all() and e.mean() < BF16_MEAN_FACTOR * mean_bar and far <= BF16_FAR_SHARE, (
-            float(e.mean()), mean_bar, far, far_bar, float(e.max()))
+        far = int((e > BF16_FAR_FACTOR * bars[2]).sum())
+        assert np.isfinite(e).all() and np.median(e) < BF16_FACTOR * bars[0] and np.quantile(e, 0.9) < BF16_TAIL_FACTOR * bars[1] \
+            and far <= max(1, BF16_FAR_SHARE * len(e)), (float(np.median(e)), float(np.quantile(e, 0.9)), far, len(e), bars, float(e.max()))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
