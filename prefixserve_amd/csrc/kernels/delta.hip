@@ -185,14 +185,78 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// One token's operands as a lane holds them while it walks: its E entries of the vectors, and the numbers.
+// SAME (the gated rule: c = p = k, one decay number per head, the removal reads the decayed state) keeps
+// k and r alone.
+template <int E, bool SAME>
+struct ScanToken {
+  float k[E], r[E], c[SAME ? 1 : E], p[SAME ? 1 : E], d[SAME ? 1 : E];
+  float ds, ps, xw, rp, rk;
+};
+
+template <int E, bool SAME>
+__device__ __forceinline__ void scan_load(ScanToken<E, SAME>& t, const float* __restrict__ vec, const float* __restrict__ sca,
+                                          const float* __restrict__ xs, int tk, int l, int col) {
+  constexpr int DP = E * kLPC, NV = SAME ? 2 : 5;
+  const float* v = vec + tk * NV * DP + l * E;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    t.k[e] = v[e];
+    t.r[e] = v[DP + e];
+    if constexpr (!SAME) {
+      t.c[e] = v[2 * DP + e];
+      t.p[e] = v[3 * DP + e];
+      t.d[e] = v[4 * DP + e];
+    }
+  }
+  const float* sc = sca + tk * 6;
+  t.ds = sc[0];
+  t.ps = sc[1];
+  t.xw = sc[2] * xs[tk * kCols + col];
+  t.rp = sc[3];
+  t.rk = sc[4];
+}
+
+// One token: the column's E entries in s, the read-out returned (the same in all 16 lanes).
+template <int E, bool SAME>
+__device__ __forceinline__ float scan_step(const ScanToken<E, SAME>& t, float (&s)[E], int reads_decayed) {
+  float dec[E];
+  float dot = 0.f, rd = 0.f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    if constexpr (SAME) {
+      dec[e] = t.ds * s[e];
+      dot = fmaf(t.k[e], dec[e], dot);
+    } else {
+      dec[e] = t.d[e] * s[e];                            // the number per head is already in the vector
+      dot = fmaf(t.c[e], reads_decayed ? dec[e] : s[e], dot);
+    }
+    rd = fmaf(t.r[e], dec[e], rd);
+  }
+  dot = row16_sum(dot);
+  rd = row16_sum(rd);
+  const float take = t.ps * dot;
+  if constexpr (SAME) {
+    const float w = take + t.xw;
+#pragma unroll
+    for (int e = 0; e < E; ++e) s[e] = fmaf(t.k[e], w, dec[e]);
+    return fmaf(w, t.rk, rd);
+  } else {
+#pragma unroll
+    for (int e = 0; e < E; ++e) s[e] = fmaf(t.k[e], t.xw, fmaf(t.p[e], take, dec[e]));
+    return fmaf(t.xw, t.rk, fmaf(take, t.rp, rd));
+  }
+}
+
 // grid (items, heads, ceil(vdim / 16)), 256 threads: column col = threadIdx.x / 16 of the block's 16,
 // lane l of its 16 holds the E entries l * E .. l * E + E - 1 of the column (dim <= 16 E). The vectors
 // of TT tokens at a time pass through LDS; the run after is already on its way from memory, in
-// registers, while a run is walked. A token costs one dependent sum over the column: with
-// dec = d * S and take = ps (c . S*), the new column is dec + p take + k xw, and its read-out
-// r . S is (r . dec) + take (r . p) + xw (r . k), where r . dec is summed beside c . S* and the two
+// registers, while a run is walked, and a token's operands are read from LDS while the token before
+// is computed. A token costs one dependent sum over the column: with dec = d * S and
+// take = ps (c . S*), the new column is dec + p take + k xw, and its read-out r . S is
+// (r . dec) + take (r . p) + xw (r . k), where r . dec is summed beside c . S* and the two
 // products of vectors alone are formed once per token for all columns when the run arrives.
-template <int E>
+template <int E, bool SAME>
 __global__ __launch_bounds__(256) void delta_scan_kernel(
     const float* __restrict__ kvec, const float* __restrict__ cvec, const float* __restrict__ pvec,
     const float* __restrict__ rvec, int64_t key_row, int heads_per_group, const float* __restrict__ dvec, int64_t dvec_row,
@@ -203,8 +267,9 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   constexpr int DP = E * kLPC;                          // the column's length, padded
   constexpr int TT = kScanRun<E>;                       // tokens per run
   constexpr int VPT = TT * DP / 256;                    // vector entries a thread carries per run
+  constexpr int NV = SAME ? 2 : 5;                      // vectors per token in LDS: k, r (, c, p, d)
   constexpr int NS = 6;                                 // numbers per token: d, ps, xs, r . p, r . k
-  __shared__ __align__(16) float vec[TT * 5 * DP];      // [TT][5][DP] k, c, p, r, d
+  __shared__ __align__(16) float vec[TT * NV * DP];
   __shared__ float sca[TT * NS];
   __shared__ float xs_[TT * kCols];
   const int item = blockIdx.x, h = blockIdx.y, g = h / heads_per_group;
@@ -216,7 +281,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
 #pragma unroll
   for (int e = 0; e < E; ++e) s[e] = (j < vdim && l * E + e < dim) ? st[e] : 0.f;
 
-  float fk[VPT], fc[VPT], fp[VPT], fr[VPT], fd[VPT], fx = 0.f, fs = 1.f;
+  float fk[VPT], fr[VPT], fc[SAME ? 1 : VPT], fp[SAME ? 1 : VPT], fd[SAME ? 1 : VPT], fx = 0.f, fs = 1.f;
   // Round tf fetches the run from token tf on into registers and walks the run before it, which the
   // round before fetched: the loads are in flight while the tokens are walked.
   for (int64_t tf = s0; tf < s1 + TT; tf += TT) {
@@ -227,12 +292,14 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
 #pragma unroll
       for (int u = 0; u < VPT; ++u) {
         const int idx = threadIdx.x + u * 256, tk = idx / DP, i = idx % DP;
-        float* v = vec + tk * 5 * DP + i;
+        float* v = vec + tk * NV * DP + i;
         v[0] = fk[u];
-        v[DP] = fc[u];
-        v[2 * DP] = fp[u];
-        v[3 * DP] = fr[u];
-        v[4 * DP] = fd[u];
+        v[DP] = fr[u];
+        if constexpr (!SAME) {
+          v[2 * DP] = fc[u];
+          v[3 * DP] = fp[u];
+          v[4 * DP] = fd[u];
+        }
       }
       if (threadIdx.x / kCols < TT) xs_[threadIdx.x] = fx;
       if (threadIdx.x < TT * 3) sca[(threadIdx.x / 3) * NS + threadIdx.x % 3] = fs;
@@ -246,10 +313,14 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
         const bool in = tk < m && i < dim;
         const int64_t at = (tf + tk) * key_row + static_cast<int64_t>(g) * dim + i;
         fk[u] = in ? kvec[at] : 0.f;
-        fc[u] = in ? cvec[at] : 0.f;
-        fp[u] = in ? pvec[at] : 0.f;
         fr[u] = in ? rvec[at] : 0.f;
-        fd[u] = (in && dvec != nullptr) ? dvec[(tf + tk) * dvec_row + static_cast<int64_t>(h) * dim + i] : 1.f;
+        if constexpr (!SAME) {
+          fc[u] = in ? cvec[at] : 0.f;
+          fp[u] = in ? pvec[at] : 0.f;
+          float d = (in && dvec != nullptr) ? dvec[(tf + tk) * dvec_row + static_cast<int64_t>(h) * dim + i] : 1.f;
+          if (in && dscal != nullptr) d *= dscal[(tf + tk) * scal_row + h];
+          fd[u] = d;
+        }
       }
       {
         const int tk = threadIdx.x / kCols, cc = threadIdx.x % kCols;
@@ -263,14 +334,14 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
     }
     if (tf == s0) continue;
     if (col < n) {                                      // r . p and r . k of token col, once for all columns
-      const float* v = vec + col * 5 * DP + l * E;
+      const float* v = vec + col * NV * DP + l * E;
       float rp = 0.f, rk = 0.f;
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        rp = fmaf(v[3 * DP + e], v[2 * DP + e], rp);
-        rk = fmaf(v[3 * DP + e], v[e], rk);
+        if constexpr (!SAME) rp = fmaf(v[DP + e], v[3 * DP + e], rp);
+        rk = fmaf(v[DP + e], v[e], rk);
       }
-      rp = row16_sum(rp);
+      if constexpr (!SAME) rp = row16_sum(rp);
       rk = row16_sum(rk);
       if (l == 0) {
         sca[col * NS + 3] = rp;
@@ -278,24 +349,19 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
       }
     }
     __syncthreads();
-    for (int tk = 0; tk < n; ++tk) {
-      const float* v = vec + tk * 5 * DP + l * E;
-      const float* sc = sca + tk * NS;
-      const float ds = sc[0], ps = sc[1], xw = sc[2] * xs_[tk * kCols + col];
-      float dec[E];
-      float dot = 0.f, rd = 0.f;
-#pragma unroll
-      for (int e = 0; e < E; ++e) {
-        dec[e] = v[4 * DP + e] * ds * s[e];
-        dot = fmaf(v[DP + e], reads_decayed ? dec[e] : s[e], dot);
-        rd = fmaf(v[3 * DP + e], dec[e], rd);
+    float* o = out + t0 * out_row + static_cast<int64_t>(h) * vdim + j;
+    const bool writes = l == 0 && j < vdim;
+    ScanToken<E, SAME> ta, tb;
+    scan_load(ta, vec, sca, xs_, 0, l, col);
+    for (int tk = 0; tk < n; tk += 2) {                 // tokens in pairs: the next one's operands are read from LDS meanwhile
+      scan_load(tb, vec, sca, xs_, min(tk + 1, TT - 1), l, col);
+      const float ra = scan_step(ta, s, reads_decayed);
+      if (writes) o[tk * out_row] = ra;
+      if (tk + 1 < n) {
+        scan_load(ta, vec, sca, xs_, min(tk + 2, TT - 1), l, col);
+        const float rb = scan_step(tb, s, reads_decayed);
+        if (writes) o[(tk + 1) * out_row] = rb;
       }
-      dot = row16_sum(dot);
-      rd = row16_sum(rd);
-      const float take = ps * dot;
-#pragma unroll
-      for (int e = 0; e < E; ++e) s[e] = fmaf(v[e], xw, fmaf(v[2 * DP + e], take, dec[e]));
-      if (l == 0 && j < vdim) out[(t0 + tk) * out_row + static_cast<int64_t>(h) * vdim + j] = fmaf(xw, sc[4], fmaf(take, sc[3], rd));
     }
   }
 #pragma unroll
@@ -331,13 +397,13 @@ __global__ __launch_bounds__(256) void heads_norm_gate_kernel(const float* __res
   }
 }
 
-template <int E>
+template <int E, bool SAME>
 static int launch_delta_scan(hipStream_t s, dim3 grid, const float* kvec, const float* cvec, const float* pvec,
                              const float* rvec, int64_t key_row, int heads_per_group, const float* dvec, int64_t dvec_row,
                              const float* dscal, const float* pscal, const float* xscal, int64_t scal_row, const float* x,
                              int64_t x_row, float* out, int64_t out_row, float* state, int64_t state_row,
                              const int32_t* item_start, const int32_t* slots, int dim, int vdim, int reads_decayed) {
-  delta_scan_kernel<E><<<grid, dim3(256), 0, s>>>(kvec, cvec, pvec, rvec, key_row, heads_per_group, dvec, dvec_row, dscal,
+  delta_scan_kernel<E, SAME><<<grid, dim3(256), 0, s>>>(kvec, cvec, pvec, rvec, key_row, heads_per_group, dvec, dvec_row, dscal,
                                                      pscal, xscal, scal_row, x, x_row, out, out_row, state, state_row,
                                                      item_start, slots, dim, vdim, reads_decayed);
   return check_launch("psamd_delta_scan");
@@ -427,8 +493,13 @@ int psamd_delta_scan(void* stream, const float* kvec, const float* cvec, const f
   while (e * kLPC < dim) e *= 2;
   const dim3 grid(static_cast<unsigned>(items), static_cast<unsigned>(heads), static_cast<unsigned>(ceil_div(vdim, kCols)));
   const int hpg = heads / key_groups;
+  // The gated rule's form: one vector serves as key, direction and removal, the decay is a number per head.
+  const bool same = cvec == kvec && pvec == kvec && dvec == nullptr && reads_decayed != 0;
 #define PSAMD_SCAN(E)                                                                                                  \
-  return launch_delta_scan<E>(s, grid, kvec, cvec, pvec, rvec, key_row, hpg, dvec, dvec_row, dscal, pscal, xscal,  \
+  return same ? launch_delta_scan<E, true>(s, grid, kvec, cvec, pvec, rvec, key_row, hpg, dvec, dvec_row, dscal, pscal, xscal,  \
+                                           scal_row, x, x_row, out, out_row, state, state_row, item_start, slots, dim, vdim,   \
+                                           reads_decayed)                                                                      \
+              : launch_delta_scan<E, false>(s, grid, kvec, cvec, pvec, rvec, key_row, hpg, dvec, dvec_row, dscal, pscal, xscal,  \
                               scal_row, x, x_row, out, out_row, state, state_row, item_start, slots, dim, vdim,        \
                               reads_decayed)
   switch (e) {
