@@ -14,8 +14,25 @@
 
 namespace psamd {
 
-// One workgroup of 256 threads per row; the row lies in LDS between its passes.
-template <typename DT, typename OT>
+// Four neighbouring values at once: a thread asks for all the memory it needs in a few wide loads that
+// are in flight together, instead of one value after the other.
+template <typename T> __device__ __forceinline__ float4 load4(const T* p);
+template <> __device__ __forceinline__ float4 load4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 load4<bf16_t>(const bf16_t* p) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xFFFF0000u), __uint_as_float(raw.y << 16),
+                     __uint_as_float(raw.y & 0xFFFF0000u));
+}
+template <typename T> __device__ __forceinline__ void store4(T* p, float4 v);
+template <> __device__ __forceinline__ void store4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
+  bf16_t q[4] = {float_to_bf16(v.x), float_to_bf16(v.y), float_to_bf16(v.z), float_to_bf16(v.w)};
+  *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(q);
+}
+
+// One workgroup of 256 threads per row; the row lies in LDS between its passes. V = 4: the width is a
+// multiple of four and every thread handles four neighbouring values at a time; V = 1: any width.
+template <typename DT, typename OT, int V>
 __global__ __launch_bounds__(256) void layernorm_step_kernel(
     float* __restrict__ residual, const int32_t* __restrict__ rows, const DT* __restrict__ delta, int n_partials,
     int64_t partial_stride, const float* __restrict__ post_w, const float* __restrict__ post_b, float post_eps,
@@ -27,41 +44,88 @@ __global__ __launch_bounds__(256) void layernorm_step_kernel(
   const int64_t src = rows != nullptr ? rows[r] : r;
   float* x = residual + src * hidden;
   const float inv_n = 1.f / static_cast<float>(hidden);
+  constexpr int kStep = 256 * V;
   if (delta != nullptr) {
     float sum = 0.f;
-    for (int i = threadIdx.x; i < hidden; i += 256) {
-      float y = 0.f;
-      for (int p = 0; p < n_partials; ++p) y += to_float<DT>(delta[p * partial_stride + r * hidden + i]);
-      row[i] = y;
-      sum += y;
+    const DT* d0 = delta + r * hidden;
+#pragma unroll 2
+    for (int i = threadIdx.x * V; i < hidden; i += kStep) {
+      if constexpr (V == 4) {
+        float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+        for (int p = 0; p < n_partials; ++p) {
+          const float4 d = load4<DT>(d0 + p * partial_stride + i);
+          y.x += d.x, y.y += d.y, y.z += d.z, y.w += d.w;
+        }
+        *reinterpret_cast<float4*>(row + i) = y;
+        sum += (y.x + y.y) + (y.z + y.w);
+      } else {
+        float y = 0.f;
+        for (int p = 0; p < n_partials; ++p) y += to_float<DT>(d0[p * partial_stride + i]);
+        row[i] = y;
+        sum += y;
+      }
     }
     const float mean = block_sum(sum, scratch, 4) * inv_n;
     float sq = 0.f;
-    for (int i = threadIdx.x; i < hidden; i += 256) {
-      const float d = row[i] - mean;
-      sq = fmaf(d, d, sq);
+    for (int i = threadIdx.x * V; i < hidden; i += kStep) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float d = row[i + e] - mean;
+        sq = fmaf(d, d, sq);
+      }
     }
     const float inv = 1.f / sqrtf(block_sum(sq, scratch, 4) * inv_n + post_eps);
-    for (int i = threadIdx.x; i < hidden; i += 256) {
-      const float v = x[i] + ((row[i] - mean) * inv * post_w[i] + post_b[i]);
-      x[i] = v;
-      row[i] = v;
+#pragma unroll 2
+    for (int i = threadIdx.x * V; i < hidden; i += kStep) {
+      if constexpr (V == 4) {
+        const float4 xv = load4<float>(x + i), w = load4<float>(post_w + i), b = load4<float>(post_b + i);
+        const float4 y = *reinterpret_cast<const float4*>(row + i);
+        const float4 v = make_float4(xv.x + ((y.x - mean) * inv * w.x + b.x), xv.y + ((y.y - mean) * inv * w.y + b.y),
+                                     xv.z + ((y.z - mean) * inv * w.z + b.z), xv.w + ((y.w - mean) * inv * w.w + b.w));
+        store4<float>(x + i, v);
+        *reinterpret_cast<float4*>(row + i) = v;
+      } else {
+        const float v = x[i] + ((row[i] - mean) * inv * post_w[i] + post_b[i]);
+        x[i] = v;
+        row[i] = v;
+      }
     }
   } else if (out != nullptr) {
-    for (int i = threadIdx.x; i < hidden; i += 256) row[i] = x[i];
+#pragma unroll 2
+    for (int i = threadIdx.x * V; i < hidden; i += kStep) {
+      if constexpr (V == 4) *reinterpret_cast<float4*>(row + i) = load4<float>(x + i);
+      else row[i] = x[i];
+    }
   }
   if (out == nullptr) return;
   float sum = 0.f;
-  for (int i = threadIdx.x; i < hidden; i += 256) sum += row[i];      // every thread reads what it wrote itself
+  for (int i = threadIdx.x * V; i < hidden; i += kStep) {             // every thread reads what it wrote itself
+#pragma unroll
+    for (int e = 0; e < V; ++e) sum += row[i + e];
+  }
   const float mean = block_sum(sum, scratch, 4) * inv_n;
   float sq = 0.f;
-  for (int i = threadIdx.x; i < hidden; i += 256) {
-    const float d = row[i] - mean;
-    sq = fmaf(d, d, sq);
+  for (int i = threadIdx.x * V; i < hidden; i += kStep) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float d = row[i + e] - mean;
+      sq = fmaf(d, d, sq);
+    }
   }
   const float inv = 1.f / sqrtf(block_sum(sq, scratch, 4) * inv_n + pre_eps);
   OT* o = out + r * hidden;
-  for (int i = threadIdx.x; i < hidden; i += 256) o[i] = from_float<OT>((row[i] - mean) * inv * pre_w[i] + pre_b[i]);
+#pragma unroll 2
+  for (int i = threadIdx.x * V; i < hidden; i += kStep) {
+    if constexpr (V == 4) {
+      const float4 w = load4<float>(pre_w + i), b = load4<float>(pre_b + i);
+      const float4 y = *reinterpret_cast<const float4*>(row + i);
+      store4<OT>(o + i, make_float4((y.x - mean) * inv * w.x + b.x, (y.y - mean) * inv * w.y + b.y,
+                                    (y.z - mean) * inv * w.z + b.z, (y.w - mean) * inv * w.w + b.w));
+    } else {
+      o[i] = from_float<OT>((row[i] - mean) * inv * pre_w[i] + pre_b[i]);
+    }
+  }
 }
 
 // x[t, e] += sin (e even) or cos (e odd) of positions[t] * freq[e / 2]. The angle is formed in double and
@@ -84,9 +148,20 @@ static int launch_layernorm(hipStream_t s, float* residual, const int32_t* rows,
                             int64_t partial_stride, const float* post_w, const float* post_b, float post_eps,
                             const float* pre_w, const float* pre_b, float pre_eps, void* out, int64_t n_rows, int hidden) {
   const size_t smem = sizeof(float) * (static_cast<size_t>(hidden) + 4);
-  layernorm_step_kernel<DT, OT><<<dim3(static_cast<unsigned>(n_rows)), dim3(256), smem, s>>>(
-      residual, rows, static_cast<const DT*>(delta), n_partials, partial_stride, post_w, post_b, post_eps, pre_w, pre_b,
-      pre_eps, static_cast<OT*>(out), hidden);
+  // Four values at a time where every row, slice and parameter starts on a multiple of four values.
+  const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool wide = hidden % 4 == 0 && partial_stride % 4 == 0 && aligned(residual) && aligned(delta) && aligned(post_w) &&
+                    aligned(post_b) && aligned(pre_w) && aligned(pre_b) && aligned(out);
+  const dim3 grid(static_cast<unsigned>(n_rows));
+  if (wide) {
+    layernorm_step_kernel<DT, OT, 4><<<grid, dim3(256), smem, s>>>(residual, rows, static_cast<const DT*>(delta), n_partials,
+                                                                  partial_stride, post_w, post_b, post_eps, pre_w, pre_b,
+                                                                  pre_eps, static_cast<OT*>(out), hidden);
+  } else {
+    layernorm_step_kernel<DT, OT, 1><<<grid, dim3(256), smem, s>>>(residual, rows, static_cast<const DT*>(delta), n_partials,
+                                                                  partial_stride, post_w, post_b, post_eps, pre_w, pre_b,
+                                                                  pre_eps, static_cast<OT*>(out), hidden);
+  }
   return check_launch("psamd_layernorm_step");
 }
 

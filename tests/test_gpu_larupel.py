@@ -83,7 +83,7 @@ def layer_norm(x, w, b, eps):
 # ------------------------------------------------------------------ kernels
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("t,h", [(1, 64), (7, 100), (130, 72), (40, 1000)])
+@pytest.mark.parametrize("t,h", [(1, 64), (7, 100), (130, 72), (40, 1000), (9, 30), (3, 2049)])
 def test_layer_norm_around_the_stream(ops, dtype, t, h):
     """stream += norm(delta) with the next norm's output from the same kernel; a delta in float32 slices;
     the norm of picked rows."""
