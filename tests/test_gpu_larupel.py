@@ -402,6 +402,23 @@ def test_sizes_at_the_kernels_limits(dtype, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_that_are_multiples_of_nothing(dtype, tmp_path):
+    """A width of 90, a vocabulary of 77, inner sizes of 50, 13 and 7, heads of 5, 9 and 11 numbers, a rank
+    of 3: the products' and the norms' narrow forms, rows that start at odd addresses."""
+    cfg = model(77, 90, 1e-6, [layer(delta(3, 1, 5, 9, 2), moe(3, 2, 13, shared=7)), layer(attention(3, 3, 11, 5, 0.4), dense(50)),
+                               layer(general_delta(2, 9, 3), moe(5, 5, 7)), layer(attention(3, 3, 11, 5, 0.4, kv_from=1), None)])
+    folder = write_larupel(tmp_path, cfg, seed=13)
+    rng = np.random.default_rng(5)
+    reqs = [rng.integers(0, 77, n).tolist() for n in (75, 40, 9)]
+    pm = plain.PlainLarupel.from_dir(folder)
+    truth = [pm.logits(t) for t in reqs]
+    steps, expect, peak = traces.mixed(reqs, max_live=3, seed=1)
+    errors: list = []
+    traces.compare(TraceReplayer(runner_for(folder, peak // 16, dtype, slots=3)).run_step, steps, expect, truth, 1.0, errors)
+    check_rows(errors, dtype, bf16_bars(folder, truth, reqs) if dtype == "bfloat16" else None)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decoding_through_graphs(dtype, folders):
     """The delta rules' kernels read slots and item boundaries from device memory, so decode steps are
     captured; the capture puts the state back before its first replay. Two requests decode side by
