@@ -33,6 +33,9 @@ constexpr int kCols = 16;     // columns per workgroup
 // Tokens whose vectors are in LDS at a time: 40 KB of vectors at most, and no more runs' worth of
 // registers per thread than eight entries of each vector.
 template <int E> constexpr int kScanRun = E == 16 ? 8 : 16;
+// Whether a whole run's tokens are written out one after the other in the code (no loop): not where a
+// lane already carries so many entries that more code in flight would not fit its registers.
+template <int E> constexpr bool kScanUnrolled = E <= 8;
 
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
 __device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
@@ -218,8 +221,8 @@ __device__ __forceinline__ void scan_load(ScanToken<E, SAME>& t, const float* __
 }
 
 // One token: the column's E entries in s, the read-out returned (the same in all 16 lanes).
-template <int E, bool SAME>
-__device__ __forceinline__ float scan_step(const ScanToken<E, SAME>& t, float (&s)[E], int reads_decayed) {
+template <int E, bool SAME, bool RD>
+__device__ __forceinline__ float scan_step(const ScanToken<E, SAME>& t, float (&s)[E]) {
   float dec[E];
   float dot = 0.f, rd = 0.f;
 #pragma unroll
@@ -229,7 +232,7 @@ __device__ __forceinline__ float scan_step(const ScanToken<E, SAME>& t, float (&
       dot = fmaf(t.k[e], dec[e], dot);
     } else {
       dec[e] = t.d[e] * s[e];                            // the number per head is already in the vector
-      dot = fmaf(t.c[e], reads_decayed ? dec[e] : s[e], dot);
+      dot = fmaf(t.c[e], RD ? dec[e] : s[e], dot);
     }
     rd = fmaf(t.r[e], dec[e], rd);
   }
@@ -248,6 +251,23 @@ __device__ __forceinline__ float scan_step(const ScanToken<E, SAME>& t, float (&
   }
 }
 
+// Tokens tk and tk + 1 of a run of n: the next token's operands are read from LDS while one is computed.
+// ta holds token tk on entry and token tk + 2 on exit.
+template <int E, bool SAME, bool RD>
+__device__ __forceinline__ void scan_two(ScanToken<E, SAME>& ta, ScanToken<E, SAME>& tb, float (&s)[E], const float* __restrict__ vec,
+                                         const float* __restrict__ sca, const float* __restrict__ xs, int tk, int n,
+                                         float* __restrict__ o, int64_t out_row, int j, bool writes, int l, int col) {
+  constexpr int TT = kScanRun<E>;
+  scan_load(tb, vec, sca, xs, min(tk + 1, TT - 1), l, col);
+  const float ra = scan_step<E, SAME, RD>(ta, s);
+  if (writes) o[tk * out_row + j] = ra;
+  if (tk + 1 < n) {
+    scan_load(ta, vec, sca, xs, min(tk + 2, TT - 1), l, col);
+    const float rb = scan_step<E, SAME, RD>(tb, s);
+    if (writes) o[(tk + 1) * out_row + j] = rb;
+  }
+}
+
 // grid (items, heads, ceil(vdim / 16)), 256 threads: column col = threadIdx.x / 16 of the block's 16,
 // lane l of its 16 holds the E entries l * E .. l * E + E - 1 of the column (dim <= 16 E). The vectors
 // of TT tokens at a time pass through LDS; the run after is already on its way from memory, in
@@ -256,14 +276,13 @@ __device__ __forceinline__ float scan_step(const ScanToken<E, SAME>& t, float (&
 // take = ps (c . S*), the new column is dec + p take + k xw, and its read-out r . S is
 // (r . dec) + take (r . p) + xw (r . k), where r . dec is summed beside c . S* and the two
 // products of vectors alone are formed once per token for all columns when the run arrives.
-template <int E, bool SAME>
+template <int E, bool SAME, bool RD>
 __global__ __launch_bounds__(256) void delta_scan_kernel(
     const float* __restrict__ kvec, const float* __restrict__ cvec, const float* __restrict__ pvec,
     const float* __restrict__ rvec, int64_t key_row, int heads_per_group, const float* __restrict__ dvec, int64_t dvec_row,
     const float* __restrict__ dscal, const float* __restrict__ pscal, const float* __restrict__ xscal, int64_t scal_row,
     const float* __restrict__ x, int64_t x_row, float* __restrict__ out, int64_t out_row, float* __restrict__ state,
-    int64_t state_row, const int32_t* __restrict__ item_start, const int32_t* __restrict__ slots, int dim, int vdim,
-    int reads_decayed) {
+    int64_t state_row, const int32_t* __restrict__ item_start, const int32_t* __restrict__ slots, int dim, int vdim) {
   constexpr int DP = E * kLPC;                          // the column's length, padded
   constexpr int TT = kScanRun<E>;                       // tokens per run
   constexpr int VPT = TT * DP / 256;                    // vector entries a thread carries per run
@@ -349,19 +368,15 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
       }
     }
     __syncthreads();
-    float* o = out + t0 * out_row + static_cast<int64_t>(h) * vdim + j;
+    float* o = out + t0 * out_row + static_cast<int64_t>(h) * vdim;   // the same in every lane: the lane's part is j
     const bool writes = l == 0 && j < vdim;
     ScanToken<E, SAME> ta, tb;
     scan_load(ta, vec, sca, xs_, 0, l, col);
-    for (int tk = 0; tk < n; tk += 2) {                 // tokens in pairs: the next one's operands are read from LDS meanwhile
-      scan_load(tb, vec, sca, xs_, min(tk + 1, TT - 1), l, col);
-      const float ra = scan_step(ta, s, reads_decayed);
-      if (writes) o[tk * out_row] = ra;
-      if (tk + 1 < n) {
-        scan_load(ta, vec, sca, xs_, min(tk + 2, TT - 1), l, col);
-        const float rb = scan_step(tb, s, reads_decayed);
-        if (writes) o[(tk + 1) * out_row] = rb;
-      }
+    if (kScanUnrolled<E> && n == TT) {                  // a whole run: every LDS address and row offset is a constant
+#pragma unroll
+      for (int tk = 0; tk < TT; tk += 2) scan_two<E, SAME, RD>(ta, tb, s, vec, sca, xs_, tk, TT, o, out_row, j, writes, l, col);
+    } else {
+      for (int tk = 0; tk < n; tk += 2) scan_two<E, SAME, RD>(ta, tb, s, vec, sca, xs_, tk, n, o, out_row, j, writes, l, col);
     }
   }
 #pragma unroll
@@ -397,15 +412,15 @@ __global__ __launch_bounds__(256) void heads_norm_gate_kernel(const float* __res
   }
 }
 
-template <int E, bool SAME>
+template <int E, bool SAME, bool RD>
 static int launch_delta_scan(hipStream_t s, dim3 grid, const float* kvec, const float* cvec, const float* pvec,
                              const float* rvec, int64_t key_row, int heads_per_group, const float* dvec, int64_t dvec_row,
                              const float* dscal, const float* pscal, const float* xscal, int64_t scal_row, const float* x,
                              int64_t x_row, float* out, int64_t out_row, float* state, int64_t state_row,
-                             const int32_t* item_start, const int32_t* slots, int dim, int vdim, int reads_decayed) {
-  delta_scan_kernel<E, SAME><<<grid, dim3(256), 0, s>>>(kvec, cvec, pvec, rvec, key_row, heads_per_group, dvec, dvec_row, dscal,
-                                                     pscal, xscal, scal_row, x, x_row, out, out_row, state, state_row,
-                                                     item_start, slots, dim, vdim, reads_decayed);
+                             const int32_t* item_start, const int32_t* slots, int dim, int vdim) {
+  delta_scan_kernel<E, SAME, RD><<<grid, dim3(256), 0, s>>>(kvec, cvec, pvec, rvec, key_row, heads_per_group, dvec, dvec_row,
+                                                           dscal, pscal, xscal, scal_row, x, x_row, out, out_row, state,
+                                                           state_row, item_start, slots, dim, vdim);
   return check_launch("psamd_delta_scan");
 }
 
@@ -495,13 +510,13 @@ int psamd_delta_scan(void* stream, const float* kvec, const float* cvec, const f
   const int hpg = heads / key_groups;
   // The gated rule's form: one vector serves as key, direction and removal, the decay is a number per head.
   const bool same = cvec == kvec && pvec == kvec && dvec == nullptr && reads_decayed != 0;
-#define PSAMD_SCAN(E)                                                                                                  \
-  return same ? launch_delta_scan<E, true>(s, grid, kvec, cvec, pvec, rvec, key_row, hpg, dvec, dvec_row, dscal, pscal, xscal,  \
-                                           scal_row, x, x_row, out, out_row, state, state_row, item_start, slots, dim, vdim,   \
-                                           reads_decayed)                                                                      \
-              : launch_delta_scan<E, false>(s, grid, kvec, cvec, pvec, rvec, key_row, hpg, dvec, dvec_row, dscal, pscal, xscal,  \
-                              scal_row, x, x_row, out, out_row, state, state_row, item_start, slots, dim, vdim,        \
-                              reads_decayed)
+#define PSAMD_SCAN_ARGS                                                                                                   \
+  s, grid, kvec, cvec, pvec, rvec, key_row, hpg, dvec, dvec_row, dscal, pscal, xscal, scal_row, x, x_row, out, out_row, state, \
+      state_row, item_start, slots, dim, vdim
+#define PSAMD_SCAN(E)                                                                                   \
+  return same ? launch_delta_scan<E, true, true>(PSAMD_SCAN_ARGS)                                       \
+              : reads_decayed ? launch_delta_scan<E, false, true>(PSAMD_SCAN_ARGS)                      \
+                              : launch_delta_scan<E, false, false>(PSAMD_SCAN_ARGS)
   switch (e) {
     case 1: PSAMD_SCAN(1);
     case 2: PSAMD_SCAN(2);
@@ -510,6 +525,7 @@ int psamd_delta_scan(void* stream, const float* kvec, const float* cvec, const f
     default: PSAMD_SCAN(16);
   }
 #undef PSAMD_SCAN
+#undef PSAMD_SCAN_ARGS
 }
 
 int psamd_heads_norm_gate(void* stream, const float* o, int64_t tokens, int heads, int vdim, const float* weight,
