@@ -174,7 +174,12 @@ class LarupelConfig:
             kind = entry.get("type")
             if kind not in MIXERS:
                 raise UnsupportedModelError(f"{where}: mixer type {kind!r}; implemented: {sorted(MIXERS)}")
-            mixer = MIXERS[kind].from_json(entry["mixer"], where + ".mixer")
+            m = entry["mixer"]
+            j = m.get("kv_from") if kind == "attention" else None
+            if isinstance(j, int) and 0 <= j < i and raw["layers"][j].get("type") == "attention":
+                # A reader's key and value sizes are its source's; a file may leave them out.
+                m = {**{k: v for k, v in raw["layers"][j]["mixer"].items() if k in ("kv_heads", "dim", "vdim")}, **m}
+            mixer = MIXERS[kind].from_json(m, where + ".mixer")
             mlp = None if entry.get("mlp") is None else _feed_forward(entry["mlp"], where + ".mlp")
             layers.append(LarupelLayer(kind, mixer, mlp))
         for i, layer in enumerate(layers):

@@ -61,6 +61,10 @@ def test_configuration_reads_every_key_and_refuses_what_it_does_not_know():
     f0, f1, f2 = (cfg.layers[i].mlp for i in range(3))
     assert (f0.experts, f0.top, f0.ff, f0.shared_ff) == (5, 2, 24, 40) and f1.ff == 80 and f2.shared_ff is None
     assert LarupelConfig.from_dicts(cfg.to_config_json()) == cfg
+    lean = copy.deepcopy(LARUPEL["A"])
+    for key in ("kv_heads", "dim", "vdim"):
+        del lean["layers"][3]["mixer"][key]                  # a reader that leaves its key sizes to its source
+    assert LarupelConfig.from_dicts(lean) == cfg
     for path, value in [(("layers", 0, "type"), "conv"), (("layers", 1, "mlp", "kind"), "glu"), (("layers", 1, "mixer", "window"), 8),
                         (("layers", 1, "mixer", "kv_heads"), 4), (("layers", 3, "mixer", "kv_from"), 2),
                         (("layers", 3, "mixer", "kv_from"), 3), (("layers", 3, "mixer", "vdim"), 8), (("layers", 0, "mlp", "router", "top"), 6),
