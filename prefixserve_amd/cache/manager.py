@@ -35,16 +35,24 @@ def blocks_for(num_tokens: int) -> int:
 
 class CacheManager:
     def __init__(self, num_blocks: Sequence[int], windows: Sequence[int | None] | None = None, num_slots: int = 64,
-                 bytes_per_slot: int = 0, enable_prefix_cache: bool = True, hash_seed: int | None = None) -> None:
+                 bytes_per_slot: int = 0, enable_prefix_cache: bool = True, hash_seed: int | None = None,
+                 keep_first: Sequence[int] | None = None, strides: Sequence[int] | None = None) -> None:
+        """``keep_first[g]``: a window group keeps the pages that hold a request's first that many
+        positions. ``strides[g]`` n: group g holds one entry per n tokens of a request (a page
+        covers 16 n tokens)."""
         self.num_groups = len(num_blocks)
         if self.num_groups < 1:
             raise ValueError("at least one layer group")
         self.windows = list(windows) if windows is not None else [None] * self.num_groups
-        if len(self.windows) != self.num_groups:
-            raise ValueError("one window entry per group")
+        self.keep_first = [int(k) for k in keep_first] if keep_first is not None else [0] * self.num_groups
+        self.strides = [int(n) for n in strides] if strides is not None else [1] * self.num_groups
+        if not len(self.windows) == len(self.keep_first) == len(self.strides) == self.num_groups:
+            raise ValueError("one window, kept-first and stride entry per group")
+        if any(n < 1 for n in self.strides) or any(k < 0 for k in self.keep_first):
+            raise ValueError("strides are at least 1 and kept positions at least 0")
         self.pools = [BlockManager(int(n)) for n in num_blocks]
         self.prefix_cache = (bool(enable_prefix_cache) and all(w is None for w in self.windows)
-                             and int(bytes_per_slot) == 0)
+                             and all(n == 1 for n in self.strides) and int(bytes_per_slot) == 0)
         self.trees = [RadixTree(p, hash_seed) for p in self.pools] if self.prefix_cache else []
         self.slots = StateSlots(int(num_slots), int(bytes_per_slot))
 
@@ -59,13 +67,17 @@ class CacheManager:
     def num_cached(self, g: int = 0) -> int:
         return self.trees[g].num_cached_blocks if self.prefix_cache else 0
 
+    def blocks_for_group(self, g: int, num_tokens: int) -> int:
+        """Entries of a block table of group g that a request of ``num_tokens`` tokens needs."""
+        return blocks_for(num_tokens // self.strides[g])
+
     def pages_needed(self, g: int, num_tokens: int, longest_step: int) -> int:
         """Most pages a request of ``num_tokens`` holds in group g at any time, when no step
         gives it more than ``longest_step`` tokens."""
         w = self.windows[g]
         if w is None:
-            return blocks_for(num_tokens)
-        return min(blocks_for(num_tokens), blocks_for(w + longest_step) + 1)
+            return self.blocks_for_group(g, num_tokens)
+        return min(blocks_for(num_tokens), blocks_for(w + longest_step) + 1 + blocks_for(self.keep_first[g]))
 
     # ------------------------------------------------------------- pages
 
@@ -124,10 +136,11 @@ class CacheManager:
             first_visible = next_position - w + 1
             last_dead_page = first_visible // BLOCK_SIZE  # pages [0, last_dead_page) lie wholly before it
             table = tables[g]
-            # Pages go back in order, so the entries already given back are a prefix of the
-            # table: walk down from the newest dead page until one of them.
+            kept = blocks_for(self.keep_first[g])         # the pages of the first positions stay
+            # Pages go back in order, so the entries already given back lie in one run behind the
+            # kept ones: walk down from the newest dead page until one of them.
             j = min(max(last_dead_page, 0), len(table)) - 1
-            while j >= 0 and table[j] >= 0:
+            while j >= kept and table[j] >= 0:
                 self.pools[g].decref(table[j])
                 table[j] = -1
                 freed += 1

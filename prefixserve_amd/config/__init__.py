@@ -1,3 +1,4 @@
+from .fubelorn import FubelornConfig
 from .gokolix import GokolixConfig
 from .larupel import LarupelConfig
 from .llama import Llama3RopeScaling, LlamaConfig, UnsupportedModelError
@@ -6,6 +7,6 @@ from .registry import (Architecture, UnknownArchitectureError, architecture_of, 
                        register_architecture, registered_architectures)
 
 __all__ = [
-    "Architecture", "GokolixConfig", "LarupelConfig", "Llama3RopeScaling", "LlamaConfig", "RadivikConfig", "UnknownArchitectureError", "UnsupportedModelError",
+    "Architecture", "FubelornConfig", "GokolixConfig", "LarupelConfig", "Llama3RopeScaling", "LlamaConfig", "RadivikConfig", "UnknownArchitectureError", "UnsupportedModelError",
     "architecture_of", "read_model_dir", "register_architecture", "registered_architectures",
 ]

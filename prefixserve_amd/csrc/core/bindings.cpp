@@ -171,10 +171,20 @@ struct Borrowed {
 // static_pages) -> None if the buffer is too small, in which case only the first number
 // of the result counts, else the layout as a tuple of integers.
 py::tuple pack_step(py::array_t<int32_t, py::array::c_style> buffer, const py::sequence& items,
-                    const std::vector<std::pair<int64_t, py::object>>& groups, int64_t vocab_size,
+                    const std::vector<py::tuple>& groups, int64_t vocab_size,
                     int64_t max_position, int64_t num_slots, int64_t prefill_tile, const py::object& static_pages) {
   std::vector<PackGroup> gs;
-  for (const auto& g : groups) gs.push_back(PackGroup{g.first, g.second.is_none() ? -1 : g.second.cast<int64_t>()});
+  for (const py::tuple& g : groups) {
+    // (pages, window or None[, kept first positions, stride])
+    if (g.size() != 2 && g.size() != 4) throw py::value_error("a group is (pages, window) or (pages, window, keep_first, stride)");
+    PackGroup pg{g[0].cast<int64_t>(), g[1].is_none() ? -1 : g[1].cast<int64_t>()};
+    if (g.size() == 4) {
+      pg.keep_first = g[2].cast<int64_t>();
+      pg.stride = g[3].cast<int64_t>();
+    }
+    if (pg.keep_first < 0 || pg.stride < 1) throw py::value_error("kept positions are at least 0 and a stride at least 1");
+    gs.push_back(pg);
+  }
   PackLimits lim;
   lim.vocab_size = vocab_size;
   lim.max_position = max_position;

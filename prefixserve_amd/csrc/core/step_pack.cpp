@@ -41,7 +41,7 @@ PackLayout plan_step(const std::vector<PackItem>& items, const std::vector<PackG
       throw PackError(i, "needs " + std::to_string(pages) + " pages, static layout has " +
                              std::to_string(lim.static_pages));
     for (size_t g = 0; g < groups.size(); ++g)
-      if (it.tables[g].size < pages)
+      if (it.tables[g].size < ceil_div(end / groups[g].stride, kBlockSize))
         throw PackError(i, std::to_string(it.tables[g].size) + " blocks in group " + std::to_string(g) + " for " +
                                std::to_string(end) + " tokens");
     lay.tokens += n;
@@ -144,15 +144,22 @@ void fill_step(const std::vector<PackItem>& items, const std::vector<PackGroup>&
       const PackItem& it = items[static_cast<size_t>(i)];
       const Span& table = it.tables[g];
       const int64_t n = it.tokens.size, end = it.start + n;
-      const int64_t pages = ceil_div(end, kBlockSize);
-      const int64_t cap = lim.static_pages >= 0 ? lim.static_pages : pages;
+      const int64_t stride = groups[g].stride;
+      // Every group's table takes as many places as the tokens' pages; a group with a stride fills fewer.
+      const int64_t token_pages = ceil_div(end, kBlockSize);
+      const int64_t pages = ceil_div(end / stride, kBlockSize);
+      const int64_t cap = lim.static_pages >= 0 ? lim.static_pages : token_pages;
       // Pages a token of this step can see or writes: all of them, or in a window group
-      // those from the window of the first new token on. Earlier entries may be -1 (given
-      // back); they are never read and go out as 0.
+      // those from the window of the first new token on and those of the kept first
+      // positions. Other earlier entries may be -1 (given back); they are never read and go out as 0.
       const int64_t first_needed =
           groups[g].window < 0 ? 0 : std::max<int64_t>(0, it.start - groups[g].window + 1) / kBlockSize;
-      for (int64_t p = 0; p < first_needed; ++p) bids[p0 + p] = 0;
-      for (int64_t p = first_needed; p < pages; ++p) {
+      const int64_t kept = groups[g].window < 0 ? 0 : std::min(ceil_div(groups[g].keep_first, kBlockSize), pages);
+      for (int64_t p = 0; p < pages; ++p) {
+        if (p >= kept && p < first_needed) {
+          bids[p0 + p] = 0;
+          continue;
+        }
         const int64_t id = table.data[p];
         if (id < 0 || id >= groups[g].num_blocks)
           throw PackError(i, "block id " + std::to_string(id) + " outside the pool of group " + std::to_string(g) +
@@ -162,7 +169,14 @@ void fill_step(const std::vector<PackItem>& items, const std::vector<PackGroup>&
       for (int64_t p = pages; p < cap; ++p) bids[p0 + p] = 0;
       for (int64_t j = 0; j < n; ++j) {
         const int64_t at = it.start + j;
-        wslot[t0 + j] = bids[p0 + at / kBlockSize] * kBlockSize + static_cast<int32_t>(at % kBlockSize);
+        if (stride == 1) {
+          wslot[t0 + j] = bids[p0 + at / kBlockSize] * kBlockSize + static_cast<int32_t>(at % kBlockSize);
+        } else if ((at + 1) % stride == 0) {       // the token that completes entry at / stride
+          const int64_t b = at / stride;
+          wslot[t0 + j] = bids[p0 + b / kBlockSize] * kBlockSize + static_cast<int32_t>(b % kBlockSize);
+        } else {
+          wslot[t0 + j] = -1;
+        }
       }
       p0 += cap;
       t0 += n;

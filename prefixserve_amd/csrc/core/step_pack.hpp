@@ -35,6 +35,8 @@ struct PackItem {
 struct PackGroup {
   int64_t num_blocks = 0;
   int64_t window = -1;  // < 0: every earlier position stays visible
+  int64_t keep_first = 0;  // a window group also keeps the pages of a request's first positions
+  int64_t stride = 1;      // the group holds one entry per `stride` tokens (entry b when token b*stride+stride-1 runs)
 };
 
 struct PackLimits {

@@ -157,6 +157,12 @@ int psamd_add_sinusoid(void* stream, float* x, const int32_t* positions, const d
 int psamd_short_conv(void* stream, const void* in, int act_dtype, int64_t in_row, const float* taps_w, float* out,
                      int64_t out_row, float* state, int64_t state_row, const int32_t* tok_item, const int32_t* item_start,
                      const int32_t* slots, int64_t tokens, int items, int channels, int taps, int act);
+// The same with a bias per channel (or NULL) added to the sum, an input of either type (in_dtype) whatever the output's,
+// and the output in out_dtype.
+int psamd_short_conv_to(void* stream, const void* in, int in_dtype, int64_t in_row, const float* taps_w, const float* bias,
+                        void* out, int out_dtype, int64_t out_row, float* state, int64_t state_row, const int32_t* tok_item,
+                        const int32_t* item_start, const int32_t* slots, int64_t tokens, int items, int channels, int taps,
+                        int act);
 // Operands of the gated delta rule: u row [q: groups x dim | k: groups x dim | ...] float, q and k made unit
 // vectors in place (q times q_scale); gates row [strength logits | decay inputs] (heads each) -> coef row
 // [g | -b | b]: b = sigmoid(.), g = exp(-exp(a_log[h]) softplus(. + dt_bias[h])).
@@ -182,6 +188,54 @@ int psamd_delta_scan(void* stream, const float* kvec, const float* cvec, const f
 int psamd_heads_norm_gate(void* stream, const float* o, int64_t tokens, int heads, int vdim, const float* weight,
                           int weight_per_head, float eps, const void* gate, int act_dtype, int64_t gate_row, int gate_act,
                           void* out);
+
+// ---- several residual streams, side-by-side mixers, recurrences through the delta scan (streams.hip) ----
+// x[r, :] <- weight * x[r, :] / sqrt(mean(x[r, :]^2) + eps), float, in place.
+int psamd_stream_rms_norm(void* stream, float* x, const float* weight, float eps, int64_t rows, int hidden);
+// out[t, :] = u / sqrt(mean(u^2) + eps) * weight (* factor), u = sum_s read[s] streams[s, t, :]; streams float
+// [count, tokens, hidden], out in out_dtype.
+int psamd_hyper_read(void* stream, const float* streams, int count, const float* read, const float* weight, float eps,
+                     const float* factor, void* out, int out_dtype, int64_t tokens, int hidden);
+// streams[t', t, :] <- sum_s mix[s, t'] streams[s, t, :] + write[t'] y[t, :], every copy from the old ones; y is one
+// tensor in delta_dtype or `slices` float slices.
+int psamd_hyper_write(void* stream, float* streams, int count, const float* mix, const float* write, const void* delta,
+                      int delta_dtype, int slices, int64_t slice_stride, int64_t tokens, int hidden);
+// out = a_scale * a + b_scale * b (float, n entries); a and b as the delta of psamd_hyper_write.
+int psamd_weighted_sum(void* stream, const void* a, int a_dtype, int a_slices, int64_t a_stride, float a_scale, const void* b,
+                       int b_dtype, int b_slices, int64_t b_stride, float b_scale, float* out, int64_t n);
+// x <- f(x) in place; kind 0 = GELU (erf), 1 = GELU (tanh form), 2 = SiLU, 3 = ReLU.
+int psamd_activation(void* stream, void* x, int act_dtype, int64_t n, int kind);
+// out = v / sqrt(mean(v^2) + eps) * weight over each of `parts` equal parts of the row, v = (y + skip[head] x) silu(gate).
+int psamd_gated_group_norm(void* stream, const float* y, const float* x, int64_t x_row, const float* skip, int heads,
+                           const void* gate, int act_dtype, int64_t gate_row, const float* weight, int parts, float eps,
+                           void* out, int64_t tokens, int inner);
+// coef row [decay | 0 | step] (heads each): step = softplus(dt + dt_bias[h]), decay = exp(-exp(a_log[h]) step).
+int psamd_state_space_prepare(void* stream, const float* dt, const float* dt_bias, const float* a_log, float* coef,
+                              int64_t tokens, int heads);
+// The exponential gates of a matrix memory with their running maximum (state[slot, h], read and left behind), item
+// by item and token by token: coef row [keep | 0 | write | exp(-m)] (heads each).
+int psamd_matrix_memory_gates(void* stream, const float* gates, const float* bias, float cap, float* coef, float* state,
+                              int64_t state_row, const int32_t* item_start, const int32_t* slots, int items, int heads);
+// u row [q * q_scale | k] float, vals row per head [v | 1] float, from rows in act_dtype.
+int psamd_matrix_memory_operands(void* stream, const void* rows, int act_dtype, int64_t in_row, int q_col, int k_col, int v_col,
+                                 int heads, int dim, int vdim, float q_scale, float* u, float* vals, int64_t tokens);
+// raw row per head [S^T q | n . q]: o = S^T q / (max(|n . q|, floor[t, h]) + read_eps), then as psamd_heads_norm_gate
+// with a weight over all heads and a sigmoid gate.
+int psamd_memory_read_norm_gate(void* stream, const float* raw, const float* floor_, int64_t floor_row, int heads, int vdim,
+                                float read_eps, const float* weight, float eps, const void* gate, int act_dtype,
+                                int64_t gate_row, void* out, int64_t tokens);
+// For every token whose pool_slot is >= 0: the mean key and value of the `block` tokens that end with it, from the
+// token pages to place pool_slot of the pool's pages (both [blocks][2][kv_heads][16 * head_dim]).
+int psamd_pool_kv_append(void* stream, const void* kv, void* pool, int act_dtype, const int32_t* positions,
+                         const int32_t* tok_item, const int32_t* table_off, const int32_t* block_ids, const int32_t* pool_slot,
+                         int64_t tokens, int hkv, int head_dim, int block);
+// Attention in a sliding window that also sees the first keep_first positions and, with pool != NULL, one mean key
+// and value per block of tokens wholly in front of the window; gate (float [tokens, hq] or NULL): output times sigmoid.
+int psamd_attention_masked(void* stream, const void* qkv, int q_stride, void* out, const void* kv, int act_dtype,
+                           int64_t tokens, const int32_t* positions, const int32_t* tok_item, const int32_t* table_off,
+                           const int32_t* block_ids, int hq, int hkv, int head_dim, float scale, int window, int keep_first,
+                           const void* pool, const int32_t* pool_table_off, const int32_t* pool_block_ids, int block,
+                           const float* gate);
 
 // out[M, N] = x[M, K] * w[N, K]^T with float accumulation (LDS-tiled FMA; exact path and fallback).
 int psamd_linear(void* stream, const void* x, int x_dtype, const void* w, int w_dtype, void* out, int out_dtype,

@@ -47,22 +47,23 @@ __device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log
 // taps - 1 tokens of an item read the inputs the state saved, and the state's saved inputs are
 // replaced by the item's last ones: both are the work of one thread per (item, channel), so that
 // nobody reads a saved input another thread has already replaced.
-template <typename A>
+template <typename A, typename O>
 __global__ __launch_bounds__(256) void short_conv_kernel(
-    const A* __restrict__ in, int64_t in_row, const float* __restrict__ w, float* __restrict__ out, int64_t out_row,
-    float* __restrict__ state, int64_t state_row, const int32_t* __restrict__ tok_item,
+    const A* __restrict__ in, int64_t in_row, const float* __restrict__ w, const float* __restrict__ bias, O* __restrict__ out,
+    int64_t out_row, float* __restrict__ state, int64_t state_row, const int32_t* __restrict__ tok_item,
     const int32_t* __restrict__ item_start, const int32_t* __restrict__ slots, int tokens, int channels, int taps, int act) {
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= channels) return;
   const int keep = taps - 1;
   const float* wc = w + static_cast<int64_t>(c) * taps;
+  const float b = bias != nullptr ? bias[c] : 0.f;
   if (static_cast<int>(blockIdx.x) < tokens) {
     const int64_t t = blockIdx.x;
     const int64_t s0 = item_start[tok_item[t]];
     if (t - s0 < keep) return;
-    float acc = 0.f;
+    float acc = b;
     for (int j = 0; j < taps; ++j) acc = fmaf(wc[j], to_float<A>(in[(t - keep + j) * in_row + c]), acc);
-    out[t * out_row + c] = act ? acc * sigmoidf_(acc) : acc;
+    out[t * out_row + c] = from_float<O>(act ? acc * sigmoidf_(acc) : acc);
     return;
   }
   const int item = static_cast<int>(blockIdx.x) - tokens;
@@ -71,13 +72,13 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
   float* saved = state + static_cast<int64_t>(slots[item]) * state_row + c;      // saved[j * channels]: oldest first
   const int first = min(n, keep);
   for (int li = 0; li < first; ++li) {
-    float acc = 0.f;
+    float acc = b;
     for (int j = 0; j < taps; ++j) {
       const int src = li - keep + j;
       const float v = src >= 0 ? to_float<A>(in[(s0 + src) * in_row + c]) : saved[static_cast<int64_t>(keep + src) * channels];
       acc = fmaf(wc[j], v, acc);
     }
-    out[(s0 + li) * out_row + c] = act ? acc * sigmoidf_(acc) : acc;
+    out[(s0 + li) * out_row + c] = from_float<O>(act ? acc * sigmoidf_(acc) : acc);
   }
   // The new saved inputs, oldest first: entry j is the input n - keep + j of the item, or a saved one
   // further back. Ascending j reads saved entries at or behind the one it writes.
@@ -430,28 +431,36 @@ using namespace psamd;
 
 extern "C" {
 
-int psamd_short_conv(void* stream, const void* in, int act_dtype, int64_t in_row, const float* taps_w, float* out,
-                     int64_t out_row, float* state, int64_t state_row, const int32_t* tok_item, const int32_t* item_start,
-                     const int32_t* slots, int64_t tokens, int items, int channels, int taps, int act) {
+int psamd_short_conv_to(void* stream, const void* in, int in_dtype, int64_t in_row, const float* taps_w, const float* bias,
+                        void* out, int out_dtype, int64_t out_row, float* state, int64_t state_row, const int32_t* tok_item,
+                        const int32_t* item_start, const int32_t* slots, int64_t tokens, int items, int channels, int taps,
+                        int act) {
   PSAMD_REQUIRE(tokens >= 0 && items >= 0 && channels > 0 && taps >= 1 && taps <= kConvMaxTaps, "bad sizes (at most 16 taps)");
   PSAMD_REQUIRE(in_row >= channels && out_row >= channels && state_row >= static_cast<int64_t>(taps - 1) * channels,
                 "rows too short");
   PSAMD_REQUIRE(tokens + items <= 2147483647LL && ceil_div(channels, 256) <= 65535, "too large for one launch");
+  PSAMD_REQUIRE((in_dtype == kBF16 || in_dtype == kF32) && (out_dtype == kBF16 || out_dtype == kF32),
+                "input and output are float32 or bfloat16");
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(tokens + items), static_cast<unsigned>(ceil_div(channels, 256)));
-  if (act_dtype == kBF16) {
-    short_conv_kernel<bf16_t><<<grid, dim3(256), 0, s>>>(static_cast<const bf16_t*>(in), in_row, taps_w, out, out_row, state,
-                                                        state_row, tok_item, item_start, slots, static_cast<int>(tokens),
-                                                        channels, taps, act);
-  } else if (act_dtype == kF32) {
-    short_conv_kernel<float><<<grid, dim3(256), 0, s>>>(static_cast<const float*>(in), in_row, taps_w, out, out_row, state,
-                                                       state_row, tok_item, item_start, slots, static_cast<int>(tokens),
-                                                       channels, taps, act);
-  } else {
-    return fail("psamd_short_conv: activation dtype must be float32 or bfloat16");
-  }
+#define PSAMD_CONV(A_, O_)                                                                                              \
+  short_conv_kernel<A_, O_><<<grid, dim3(256), 0, s>>>(static_cast<const A_*>(in), in_row, taps_w, bias,               \
+                                                       static_cast<O_*>(out), out_row, state, state_row, tok_item,     \
+                                                       item_start, slots, static_cast<int>(tokens), channels, taps, act)
+  if (in_dtype == kBF16 && out_dtype == kF32) PSAMD_CONV(bf16_t, float);
+  else if (in_dtype == kF32 && out_dtype == kF32) PSAMD_CONV(float, float);
+  else if (in_dtype == kF32 && out_dtype == kBF16) PSAMD_CONV(float, bf16_t);
+  else PSAMD_CONV(bf16_t, bf16_t);
+#undef PSAMD_CONV
   return check_launch("psamd_short_conv");
+}
+
+int psamd_short_conv(void* stream, const void* in, int act_dtype, int64_t in_row, const float* taps_w, float* out,
+                     int64_t out_row, float* state, int64_t state_row, const int32_t* tok_item, const int32_t* item_start,
+                     const int32_t* slots, int64_t tokens, int items, int channels, int taps, int act) {
+  return psamd_short_conv_to(stream, in, act_dtype, in_row, taps_w, nullptr, out, kF32, out_row, state, state_row, tok_item,
+                             item_start, slots, tokens, items, channels, taps, act);
 }
 
 int psamd_gated_delta_prepare(void* stream, float* u, int64_t u_row, int groups, int dim, const float* gates,

@@ -1,0 +1,417 @@
+// Several copies of the residual stream, mixers side by side, a feed-forward without a gate, and the
+// operands of two recurrences that run through the delta rules' scan:
+//   * stream_rms_norm: an RMS norm on float rows in place;
+//   * hyper_read / hyper_write: a sub-layer reads a weighted sum of the copies through an RMS norm and
+//     writes every copy from a mix of the old ones plus its own output;
+//   * weighted_sum: a * x + b * y of two sub-layer outputs (each one tensor or float slices);
+//   * activation: an elementwise function in place;
+//   * gated_group_norm: (y + skip x) silu(z), an RMS norm in equal parts, a weight;
+//   * state_space_prepare: step size and decay of a selective state space layer;
+//   * matrix_memory_gates / _operands / memory_read_norm_gate: a matrix memory's exponential gates with
+//     their running maximum, its operands as float vectors, and its read-out behind the scan;
+//   * pool_kv_append: the mean key and value of a block of tokens, written to a page of its own.
+// Everything here is float arithmetic; rows in the activation type are widened when read.
+
+#include "api.h"
+#include "common.h"
+
+namespace psamd {
+
+constexpr int kMaxStreams = 16;
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// grid (rows), 256 threads.
+__global__ __launch_bounds__(256) void stream_rms_norm_kernel(float* __restrict__ x, const float* __restrict__ w, float eps,
+                                                              int hidden) {
+  __shared__ float scratch[4];
+  float* row = x + static_cast<int64_t>(blockIdx.x) * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += 256) ss = fmaf(row[i], row[i], ss);
+  ss = block_sum(ss, scratch, 4);
+  const float inv = 1.f / sqrtf(ss / static_cast<float>(hidden) + eps);
+  for (int i = threadIdx.x; i < hidden; i += 256) row[i] = row[i] * inv * w[i];
+}
+
+// grid (tokens), 256 threads: u = sum_s read[s] streams[s, t, :]; out = u / rms(u) * w (* factor).
+template <typename O>
+__global__ __launch_bounds__(256) void hyper_read_kernel(const float* __restrict__ streams, int64_t stream_stride, int count,
+                                                         const float* __restrict__ read, const float* __restrict__ w, float eps,
+                                                         const float* __restrict__ factor, O* __restrict__ out, int hidden) {
+  __shared__ float scratch[4];
+  const float* base = streams + static_cast<int64_t>(blockIdx.x) * hidden;
+  float a[kMaxStreams];
+#pragma unroll
+  for (int s = 0; s < kMaxStreams; ++s) a[s] = s < count ? read[s] : 0.f;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < kMaxStreams; ++s)
+      if (s < count) u = fmaf(a[s], base[s * stream_stride + i], u);
+    ss = fmaf(u, u, ss);
+  }
+  ss = block_sum(ss, scratch, 4);
+  const float inv = 1.f / sqrtf(ss / static_cast<float>(hidden) + eps);
+  O* o = out + static_cast<int64_t>(blockIdx.x) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < kMaxStreams; ++s)
+      if (s < count) u = fmaf(a[s], base[s * stream_stride + i], u);
+    float v = u * inv * w[i];
+    if (factor != nullptr) v *= factor[i];
+    o[i] = from_float<O>(v);
+  }
+}
+
+// One thread per (token, channel): new[t] = sum_s mix[s, t] old[s] + write[t] * y, y = the delta (one
+// tensor in delta_dtype, or `slices` float slices slice_stride apart, added in ascending order).
+__global__ __launch_bounds__(256) void hyper_write_kernel(float* __restrict__ streams, int64_t stream_stride, int count,
+                                                          const float* __restrict__ mix, const float* __restrict__ write,
+                                                          const void* __restrict__ delta, int delta_dtype, int slices,
+                                                          int64_t slice_stride, int64_t n) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= n) return;
+  float y;
+  if (slices > 1 || delta_dtype == kF32) {
+    const float* d = static_cast<const float*>(delta);
+    y = d[e];
+    for (int s = 1; s < slices; ++s) y += d[s * slice_stride + e];
+  } else {
+    y = bf16_to_float(static_cast<const bf16_t*>(delta)[e]);
+  }
+  float old[kMaxStreams];
+#pragma unroll
+  for (int s = 0; s < kMaxStreams; ++s) old[s] = s < count ? streams[s * stream_stride + e] : 0.f;
+#pragma unroll
+  for (int t = 0; t < kMaxStreams; ++t) {
+    if (t < count) {
+      float v = write[t] * y;
+#pragma unroll
+      for (int s = 0; s < kMaxStreams; ++s)
+        if (s < count) v = fmaf(mix[s * count + t], old[s], v);
+      streams[t * stream_stride + e] = v;
+    }
+  }
+}
+
+__device__ __forceinline__ float delta_at(const void* d, int dtype, int slices, int64_t stride, int64_t e) {
+  if (slices > 1 || dtype == kF32) {
+    const float* f = static_cast<const float*>(d);
+    float y = f[e];
+    for (int s = 1; s < slices; ++s) y += f[s * stride + e];
+    return y;
+  }
+  return bf16_to_float(static_cast<const bf16_t*>(d)[e]);
+}
+
+__global__ __launch_bounds__(256) void weighted_sum_kernel(const void* __restrict__ a, int a_dtype, int a_slices, int64_t a_stride,
+                                                           float a_scale, const void* __restrict__ b, int b_dtype, int b_slices,
+                                                           int64_t b_stride, float b_scale, float* __restrict__ out, int64_t n) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= n) return;
+  out[e] = fmaf(a_scale, delta_at(a, a_dtype, a_slices, a_stride, e), b_scale * delta_at(b, b_dtype, b_slices, b_stride, e));
+}
+
+// kind 0 = GELU (exact), 1 = GELU (tanh form), 2 = SiLU, 3 = ReLU.
+template <typename A>
+__global__ __launch_bounds__(256) void activation_kernel(A* __restrict__ x, int64_t n, int kind) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= n) return;
+  const float z = to_float<A>(x[e]);
+  float v;
+  if (kind == 0) v = 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
+  else if (kind == 1) v = gelu_tanh_f(z);
+  else if (kind == 2) v = z * sigmoid_f(z);
+  else v = fmaxf(z, 0.f);
+  x[e] = from_float<A>(v);
+}
+
+// One wave per (token, part): v = (y + skip[head] x) * silu(z); out = v / sqrt(mean(v^2) + eps) * weight.
+template <typename A>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, const float* __restrict__ x,
+                                                               int64_t x_row, const float* __restrict__ skip, int vdim,
+                                                               const A* __restrict__ gate, int64_t gate_row,
+                                                               const float* __restrict__ weight, int parts, int part, float eps,
+                                                               A* __restrict__ out, int64_t pairs) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t pair = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int64_t t = pair / parts;
+  const int c0 = static_cast<int>(pair - t * parts) * part;
+  const int64_t inner = static_cast<int64_t>(parts) * part;
+  float ss = 0.f;
+  for (int i = lane; i < part; i += kWave) {
+    const int c = c0 + i;
+    const float z = to_float<A>(gate[t * gate_row + c]);
+    const float v = fmaf(skip[c / vdim], x[t * x_row + c], y[t * inner + c]) * z * sigmoid_f(z);
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / static_cast<float>(part) + eps);
+  for (int i = lane; i < part; i += kWave) {
+    const int c = c0 + i;
+    const float z = to_float<A>(gate[t * gate_row + c]);
+    const float v = fmaf(skip[c / vdim], x[t * x_row + c], y[t * inner + c]) * z * sigmoid_f(z);
+    out[t * inner + c] = from_float<A>(v * inv * weight[c]);
+  }
+}
+
+// coef row = [exp(-exp(a_log[h]) d) | 0 | d], d = softplus(dt[t, h] + dt_bias[h]).
+__global__ __launch_bounds__(256) void state_space_prepare_kernel(const float* __restrict__ dt, const float* __restrict__ dt_bias,
+                                                                  const float* __restrict__ a_log, float* __restrict__ coef,
+                                                                  int64_t n, int heads) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= n) return;
+  const int64_t t = e / heads;
+  const int h = static_cast<int>(e - t * heads);
+  const float d = softplus_f(dt[e] + dt_bias[h]);
+  float* c = coef + t * 3 * heads;
+  c[h] = expf(-expf(a_log[h]) * d);
+  c[heads + h] = 0.f;
+  c[2 * heads + h] = d;
+}
+
+// grid (items), threads over heads: the gates of a matrix memory with their running maximum m, token by
+// token. gates row = [input | forget] inputs (heads each); i = cap tanh((. + b) / cap), f = logsigmoid(cap tanh(.));
+// m' = max(f + m, i); coef row = [exp(f + m - m') | 0 | exp(i - m') | exp(-m')]; m lives in the item's slot.
+__global__ __launch_bounds__(64) void matrix_memory_gates_kernel(const float* __restrict__ gates, const float* __restrict__ bias,
+                                                                 float cap, float* __restrict__ coef, float* __restrict__ state,
+                                                                 int64_t state_row, const int32_t* __restrict__ item_start,
+                                                                 const int32_t* __restrict__ slots, int heads) {
+  const int item = blockIdx.x;
+  const int64_t s0 = item_start[item], s1 = item_start[item + 1];
+  for (int h = threadIdx.x; h < heads; h += blockDim.x) {
+    float* mp = state + static_cast<int64_t>(slots[item]) * state_row + h;
+    float m = *mp;
+    const float bi = bias[h], bf = bias[heads + h];
+    for (int64_t t = s0; t < s1; ++t) {
+      const float il = cap * tanhf((gates[t * 2 * heads + h] + bi) / cap);
+      const float fl = -softplus_f(-cap * tanhf((gates[t * 2 * heads + heads + h] + bf) / cap));
+      const float mn = fmaxf(fl + m, il);
+      float* c = coef + t * 4 * heads;
+      c[h] = expf(fl + m - mn);
+      c[heads + h] = 0.f;
+      c[2 * heads + h] = expf(il - mn);
+      c[3 * heads + h] = expf(-mn);
+      m = mn;
+    }
+    *mp = m;
+  }
+}
+
+// grid (tokens), 256 threads: u row = [q * q_scale | k] (heads x dim each), vals row = per head [v | 1].
+template <typename A>
+__global__ __launch_bounds__(256) void matrix_memory_operands_kernel(const A* __restrict__ rows, int64_t in_row, int q_col, int k_col,
+                                                                     int v_col, int heads, int dim, int vdim, float q_scale,
+                                                                     float* __restrict__ u, float* __restrict__ vals) {
+  const int64_t t = blockIdx.x;
+  const A* r = rows + t * in_row;
+  const int hd = heads * dim;
+  for (int i = threadIdx.x; i < hd; i += 256) {
+    u[t * 2 * hd + i] = to_float<A>(r[q_col + i]) * q_scale;
+    u[t * 2 * hd + hd + i] = to_float<A>(r[k_col + i]);
+  }
+  const int hv = heads * (vdim + 1);
+  for (int i = threadIdx.x; i < hv; i += 256) {
+    const int h = i / (vdim + 1), j = i - h * (vdim + 1);
+    vals[t * hv + i] = j < vdim ? to_float<A>(r[v_col + h * vdim + j]) : 1.f;
+  }
+}
+
+// One wave per (token, head): raw = [S^T q : vdim | n . q]; o = raw / (max(|n . q|, floor) + read_eps);
+// out = o / sqrt(mean(o^2) + eps) * weight[h, :] * sigmoid(gate).
+template <typename A>
+__global__ __launch_bounds__(256) void memory_read_norm_gate_kernel(const float* __restrict__ raw, const float* __restrict__ floor_,
+                                                                    int64_t floor_row, int heads, int vdim, float read_eps,
+                                                                    const float* __restrict__ weight, float eps,
+                                                                    const A* __restrict__ gate, int64_t gate_row,
+                                                                    A* __restrict__ out, int64_t pairs) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t pair = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int64_t t = pair / heads;
+  const int h = static_cast<int>(pair - t * heads);
+  const float* src = raw + pair * (vdim + 1);
+  const float den = fmaxf(fabsf(src[vdim]), floor_[t * floor_row + h]) + read_eps;
+  float ss = 0.f;
+  for (int i = lane; i < vdim; i += kWave) {
+    const float o = src[i] / den;
+    ss = fmaf(o, o, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / static_cast<float>(vdim) + eps);
+  for (int i = lane; i < vdim; i += kWave) {
+    const float z = to_float<A>(gate[t * gate_row + static_cast<int64_t>(h) * vdim + i]);
+    out[pair * vdim + i] = from_float<A>(src[i] / den * inv * weight[static_cast<int64_t>(h) * vdim + i] * sigmoid_f(z));
+  }
+}
+
+// grid (tokens, kv heads), 64 threads. A token whose pool_slot is >= 0 completes a block of `block`
+// tokens: the mean of their keys ([16][d] halves of the token pages) and values ([d][16]) goes to
+// place pool_slot of the pool's pages, summed in float in the order of the positions.
+template <typename A>
+__global__ __launch_bounds__(64) void pool_kv_append_kernel(const A* __restrict__ kv, A* __restrict__ pool,
+                                                            const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_item,
+                                                            const int32_t* __restrict__ table_off, const int32_t* __restrict__ block_ids,
+                                                            const int32_t* __restrict__ pool_slot, int hkv, int d, int block) {
+  const int64_t t = blockIdx.x;
+  const int slot = pool_slot[t];
+  if (slot < 0) return;
+  const int kvh = blockIdx.y;
+  const int pos = positions[t];
+  const int32_t* table = block_ids + table_off[tok_item[t]];
+  const int64_t page_elems = 2LL * hkv * kPage * d, half = static_cast<int64_t>(hkv) * kPage * d;
+  const float inv = 1.f / static_cast<float>(block);
+  A* dst = pool + static_cast<int64_t>(slot / kPage) * page_elems + static_cast<int64_t>(kvh) * kPage * d;
+  const int off = slot % kPage;
+  for (int i = threadIdx.x; i < d; i += kWave) {
+    float ks = 0.f, vs = 0.f;
+    for (int j = pos - block + 1; j <= pos; ++j) {
+      const A* src = kv + static_cast<int64_t>(table[j / kPage]) * page_elems + static_cast<int64_t>(kvh) * kPage * d;
+      ks += to_float<A>(src[(j % kPage) * d + i]);
+      vs += to_float<A>(src[half + static_cast<int64_t>(i) * kPage + (j % kPage)]);
+    }
+    dst[off * d + i] = from_float<A>(ks * inv);
+    dst[half + static_cast<int64_t>(i) * kPage + off] = from_float<A>(vs * inv);
+  }
+}
+
+}  // namespace psamd
+
+using namespace psamd;
+
+#define PSAMD_BY_DTYPE(code, CALL)                                                   \
+  if ((code) == kBF16) { using A_ = bf16_t; CALL; }                                  \
+  else if ((code) == kF32) { using A_ = float; CALL; }                               \
+  else return fail(std::string(__func__) + ": dtype must be float32 or bfloat16")
+
+extern "C" {
+
+int psamd_stream_rms_norm(void* stream, float* x, const float* weight, float eps, int64_t rows, int hidden) {
+  PSAMD_REQUIRE(rows >= 0 && rows <= 2147483647LL && hidden > 0, "bad sizes");
+  if (rows == 0) return 0;
+  stream_rms_norm_kernel<<<dim3(static_cast<unsigned>(rows)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(x, weight, eps, hidden);
+  return check_launch("psamd_stream_rms_norm");
+}
+
+int psamd_hyper_read(void* stream, const float* streams, int count, const float* read, const float* weight, float eps,
+                     const float* factor, void* out, int out_dtype, int64_t tokens, int hidden) {
+  PSAMD_REQUIRE(tokens >= 0 && tokens <= 2147483647LL && hidden > 0 && count >= 1 && count <= kMaxStreams, "bad sizes (at most 16 streams)");
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t stride = tokens * hidden;
+  PSAMD_BY_DTYPE(out_dtype, (hyper_read_kernel<A_><<<dim3(static_cast<unsigned>(tokens)), dim3(256), 0, s>>>(
+                                streams, stride, count, read, weight, eps, factor, static_cast<A_*>(out), hidden)));
+  return check_launch("psamd_hyper_read");
+}
+
+int psamd_hyper_write(void* stream, float* streams, int count, const float* mix, const float* write, const void* delta,
+                      int delta_dtype, int slices, int64_t slice_stride, int64_t tokens, int hidden) {
+  PSAMD_REQUIRE(tokens >= 0 && hidden > 0 && count >= 1 && count <= kMaxStreams && slices >= 1, "bad sizes (at most 16 streams)");
+  PSAMD_REQUIRE(delta_dtype == kF32 || (delta_dtype == kBF16 && slices == 1), "the delta is one tensor or float slices");
+  const int64_t n = tokens * hidden;
+  if (n == 0) return 0;
+  PSAMD_REQUIRE(ceil_div(n, 256) <= 2147483647LL, "too large for one launch");
+  hyper_write_kernel<<<dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      streams, n, count, mix, write, delta, delta_dtype, slices, slice_stride, n);
+  return check_launch("psamd_hyper_write");
+}
+
+int psamd_weighted_sum(void* stream, const void* a, int a_dtype, int a_slices, int64_t a_stride, float a_scale, const void* b,
+                       int b_dtype, int b_slices, int64_t b_stride, float b_scale, float* out, int64_t n) {
+  PSAMD_REQUIRE(n >= 0 && a_slices >= 1 && b_slices >= 1, "bad sizes");
+  PSAMD_REQUIRE((a_dtype == kF32 || (a_dtype == kBF16 && a_slices == 1)) && (b_dtype == kF32 || (b_dtype == kBF16 && b_slices == 1)),
+                "an operand is one tensor or float slices");
+  if (n == 0) return 0;
+  PSAMD_REQUIRE(ceil_div(n, 256) <= 2147483647LL, "too large for one launch");
+  weighted_sum_kernel<<<dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      a, a_dtype, a_slices, a_stride, a_scale, b, b_dtype, b_slices, b_stride, b_scale, out, n);
+  return check_launch("psamd_weighted_sum");
+}
+
+int psamd_activation(void* stream, void* x, int act_dtype, int64_t n, int kind) {
+  PSAMD_REQUIRE(n >= 0 && kind >= 0 && kind <= 3, "bad size or activation");
+  if (n == 0) return 0;
+  PSAMD_REQUIRE(ceil_div(n, 256) <= 2147483647LL, "too large for one launch");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  PSAMD_BY_DTYPE(act_dtype, (activation_kernel<A_><<<dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, s>>>(
+                                static_cast<A_*>(x), n, kind)));
+  return check_launch("psamd_activation");
+}
+
+int psamd_gated_group_norm(void* stream, const float* y, const float* x, int64_t x_row, const float* skip, int heads,
+                           const void* gate, int act_dtype, int64_t gate_row, const float* weight, int parts, float eps,
+                           void* out, int64_t tokens, int inner) {
+  PSAMD_REQUIRE(tokens >= 0 && inner > 0 && heads > 0 && parts > 0 && inner % heads == 0 && inner % parts == 0, "bad sizes");
+  const int64_t pairs = tokens * parts;
+  if (pairs == 0) return 0;
+  PSAMD_REQUIRE(ceil_div(pairs, 4) <= 2147483647LL, "too large for one launch");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  PSAMD_BY_DTYPE(act_dtype, (gated_group_norm_kernel<A_><<<dim3(static_cast<unsigned>(ceil_div(pairs, 4))), dim3(256), 0, s>>>(
+                                y, x, x_row, skip, inner / heads, static_cast<const A_*>(gate), gate_row, weight, parts,
+                                inner / parts, eps, static_cast<A_*>(out), pairs)));
+  return check_launch("psamd_gated_group_norm");
+}
+
+int psamd_state_space_prepare(void* stream, const float* dt, const float* dt_bias, const float* a_log, float* coef,
+                              int64_t tokens, int heads) {
+  PSAMD_REQUIRE(tokens >= 0 && heads > 0, "bad sizes");
+  const int64_t n = tokens * heads;
+  if (n == 0) return 0;
+  state_space_prepare_kernel<<<dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      dt, dt_bias, a_log, coef, n, heads);
+  return check_launch("psamd_state_space_prepare");
+}
+
+int psamd_matrix_memory_gates(void* stream, const float* gates, const float* bias, float cap, float* coef, float* state,
+                              int64_t state_row, const int32_t* item_start, const int32_t* slots, int items, int heads) {
+  PSAMD_REQUIRE(items >= 0 && heads > 0 && cap > 0.f && state_row >= heads, "bad sizes");
+  if (items == 0) return 0;
+  matrix_memory_gates_kernel<<<dim3(static_cast<unsigned>(items)), dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+      gates, bias, cap, coef, state, state_row, item_start, slots, heads);
+  return check_launch("psamd_matrix_memory_gates");
+}
+
+int psamd_matrix_memory_operands(void* stream, const void* rows, int act_dtype, int64_t in_row, int q_col, int k_col, int v_col,
+                                 int heads, int dim, int vdim, float q_scale, float* u, float* vals, int64_t tokens) {
+  PSAMD_REQUIRE(tokens >= 0 && tokens <= 2147483647LL && heads > 0 && dim > 0 && vdim > 0, "bad sizes");
+  PSAMD_REQUIRE(std::min(std::min(q_col, k_col), v_col) >= 0 && std::max(q_col, k_col) + static_cast<int64_t>(heads) * dim <= in_row &&
+                    v_col + static_cast<int64_t>(heads) * vdim <= in_row, "columns outside the rows");
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  PSAMD_BY_DTYPE(act_dtype, (matrix_memory_operands_kernel<A_><<<dim3(static_cast<unsigned>(tokens)), dim3(256), 0, s>>>(
+                                static_cast<const A_*>(rows), in_row, q_col, k_col, v_col, heads, dim, vdim, q_scale, u, vals)));
+  return check_launch("psamd_matrix_memory_operands");
+}
+
+int psamd_memory_read_norm_gate(void* stream, const float* raw, const float* floor_, int64_t floor_row, int heads, int vdim,
+                                float read_eps, const float* weight, float eps, const void* gate, int act_dtype,
+                                int64_t gate_row, void* out, int64_t tokens) {
+  PSAMD_REQUIRE(tokens >= 0 && heads > 0 && vdim > 0, "bad sizes");
+  const int64_t pairs = tokens * heads;
+  if (pairs == 0) return 0;
+  PSAMD_REQUIRE(ceil_div(pairs, 4) <= 2147483647LL, "too large for one launch");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  PSAMD_BY_DTYPE(act_dtype, (memory_read_norm_gate_kernel<A_><<<dim3(static_cast<unsigned>(ceil_div(pairs, 4))), dim3(256), 0, s>>>(
+                                raw, floor_, floor_row, heads, vdim, read_eps, weight, eps, static_cast<const A_*>(gate),
+                                gate_row, static_cast<A_*>(out), pairs)));
+  return check_launch("psamd_memory_read_norm_gate");
+}
+
+int psamd_pool_kv_append(void* stream, const void* kv, void* pool, int act_dtype, const int32_t* positions,
+                         const int32_t* tok_item, const int32_t* table_off, const int32_t* block_ids, const int32_t* pool_slot,
+                         int64_t tokens, int hkv, int head_dim, int block) {
+  PSAMD_REQUIRE(tokens >= 0 && tokens <= 2147483647LL && hkv > 0 && hkv <= 65535 && head_dim > 0 && block >= 1, "bad sizes");
+  if (tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(tokens), static_cast<unsigned>(hkv));
+  PSAMD_BY_DTYPE(act_dtype, (pool_kv_append_kernel<A_><<<grid, dim3(64), 0, s>>>(
+                                static_cast<const A_*>(kv), static_cast<A_*>(pool), positions, tok_item, table_off, block_ids,
+                                pool_slot, hkv, head_dim, block)));
+  return check_launch("psamd_pool_kv_append");
+}
+
+}  // extern "C"

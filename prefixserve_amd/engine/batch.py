@@ -44,13 +44,16 @@ class StepItem:
 class GroupMeta:
     num_blocks: int
     window: int | None = None
+    keep_first: int = 0     # a window group keeps the pages of a request's first positions
+    stride: int = 1         # one entry per this many tokens
 
 
 @dataclass
 class GroupArrays:
     table_off: torch.Tensor    # [B+1] start of each item's table in block_ids
     block_ids: torch.Tensor    # [P]
-    write_slot: torch.Tensor   # [T]   page * 16 + offset where each new token's K/V goes
+    write_slot: torch.Tensor   # [T]   page * 16 + offset where each new token's K/V goes (a group with a stride: the
+                               #       entry the token completes, or -1)
     table_off_host: np.ndarray
     block_ids_host: np.ndarray
 
@@ -110,7 +113,8 @@ class StepPacker:
         self.on_gpu = self.device.type == "cuda"
         self._copied = torch.cuda.Event() if self.on_gpu else None
         self._pack_step = ensure_core().pack_step
-        self._group_args = [(int(g.num_blocks), None if g.window is None else int(g.window)) for g in self.groups]
+        self._group_args = [(int(g.num_blocks), None if g.window is None else int(g.window), int(g.keep_first), int(g.stride))
+                            for g in self.groups]
         self._alloc(capacity)
 
     def _alloc(self, capacity: int) -> None:

@@ -81,7 +81,7 @@ class Engine:
         """The host-side manager of exactly this engine's pools and slots."""
         r = self.runner
         return CacheManager(r.num_blocks_per_group, r.windows, r.max_num_seqs, r.state_bytes_per_slot,
-                            enable_prefix_cache=enable_prefix_cache)
+                            enable_prefix_cache=enable_prefix_cache, keep_first=r.keep_first, strides=r.strides)
 
     def make_scheduler(self, *, max_waiting: int = 1024, chunk_size: int | None = None,
                        enable_prefix_cache: bool = True) -> Scheduler:

@@ -16,7 +16,7 @@ from typing import Any, Mapping
 
 import numpy as np
 
-from prefixserve_amd.cache.manager import CacheManager, blocks_for
+from prefixserve_amd.cache.manager import CacheManager
 from prefixserve_amd.engine.batch import EngineError, StepItem
 from prefixserve_amd.engine.runner import ModelRunner
 
@@ -36,7 +36,7 @@ class TraceReplayer:
         # skipped. Pages still come from the real allocator and are used again once freed.
         self.cache = cache if cache is not None else CacheManager(
             runner.num_blocks_per_group, runner.windows, runner.max_num_seqs, runner.state_bytes_per_slot,
-            enable_prefix_cache=False)
+            enable_prefix_cache=False, keep_first=runner.keep_first, strides=runner.strides)
         self.live: dict[Any, _Live] = {}
 
     def run_step(self, step: Mapping[str, Any]) -> np.ndarray | None:
@@ -59,7 +59,7 @@ class TraceReplayer:
                     raise EngineError(f"no free state slot for request {rid!r}")
                 st = _Live(slot=slot, tables=[[] for _ in range(self.cache.num_groups)])
                 self.live[rid] = st
-            need = [blocks_for(st.length + len(toks)) - len(t) for t in st.tables]
+            need = [self.cache.blocks_for_group(g, st.length + len(toks)) - len(t) for g, t in enumerate(st.tables)]
             fresh = self.cache.allocate([max(n, 0) for n in need])
             if fresh is None:
                 raise EngineError(f"out of pages: request {rid!r} needs {need} more; --max-tokens is too small")

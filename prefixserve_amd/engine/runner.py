@@ -96,7 +96,8 @@ class ModelRunner:
         self.pools = KVPools(self.layer_groups, self.num_blocks_per_group, self.dtype, self.device)
         self.model.attach(self.pools.layer_caches(), self.states)
         self.packer = StepPacker(
-            self.device, [GroupMeta(nb, g.need.window) for g, nb in zip(self.layer_groups, blocks)],
+            self.device, [GroupMeta(nb, g.need.window, g.need.keep_first, g.need.stride)
+                          for g, nb in zip(self.layer_groups, blocks)],
             self.spec.vocab_size, self.max_seq_len, self.max_num_seqs, self.ops.PREFILL_TILE_Q,
             skew_rule=getattr(self.ops, "decode_is_skewed", None))
 
@@ -110,6 +111,14 @@ class ModelRunner:
     @property
     def windows(self) -> list[int | None]:
         return [g.need.window for g in self.layer_groups]
+
+    @property
+    def keep_first(self) -> list[int]:
+        return [g.need.keep_first for g in self.layer_groups]
+
+    @property
+    def strides(self) -> list[int]:
+        return [g.need.stride for g in self.layer_groups]
 
     @property
     def stop_token_ids(self) -> frozenset[int]:

@@ -229,7 +229,7 @@ class Scheduler:
     def _grow(self, req: Request, upto: int, plan: _Plan) -> bool:
         """Pages for positions [0, upto) of a running request. False: ``req`` itself had to go."""
         while True:
-            short = [max(blocks_for(upto) - len(table), 0) for table in req.block_tables]
+            short = [max(self.cache.blocks_for_group(g, upto) - len(table), 0) for g, table in enumerate(req.block_tables)]
             if not any(short):
                 return True
             fresh = self.cache.allocate(short)
@@ -251,7 +251,7 @@ class Scheduler:
         slot = self.cache.acquire_slot() if count > 0 else None
         own = None
         if slot is not None:
-            own = self.cache.allocate([blocks_for(hit + count) - len(table) for table in shared])
+            own = self.cache.allocate([self.cache.blocks_for_group(g, hit + count) - len(table) for g, table in enumerate(shared)])
         if own is None:
             self.cache.release(shared)
             if slot is not None:
@@ -288,7 +288,7 @@ class Scheduler:
             return 1
         for item in plan.items:
             tables = item.req.block_tables
-            short = [max(blocks_for(item.start + steps) - len(table), 0) for table in tables]
+            short = [max(self.cache.blocks_for_group(g, item.start + steps) - len(table), 0) for g, table in enumerate(tables)]
             if any(short):
                 fresh = self.cache.allocate(short)
                 if fresh is None:

@@ -102,7 +102,23 @@ _SIGNATURES = {
     "psamd_delta_scan": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64,
                          _vp, _vp, _i32, _i32, _i32, _i32, _i32],
     "psamd_heads_norm_gate": [_vp, _vp, _i64, _i32, _i32, _vp, _i32, _f32, _vp, _i32, _i64, _i32, _vp],
+    "psamd_short_conv_to": [_vp, _vp, _i32, _i64, _vp, _vp, _vp, _i32, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32],
+    "psamd_stream_rms_norm": [_vp, _vp, _vp, _f32, _i64, _i32],
+    "psamd_hyper_read": [_vp, _vp, _i32, _vp, _vp, _f32, _vp, _vp, _i32, _i64, _i32],
+    "psamd_hyper_write": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i64, _i64, _i32],
+    "psamd_weighted_sum": [_vp, _vp, _i32, _i32, _i64, _f32, _vp, _i32, _i32, _i64, _f32, _vp, _i64],
+    "psamd_activation": [_vp, _vp, _i32, _i64, _i32],
+    "psamd_gated_group_norm": [_vp, _vp, _vp, _i64, _vp, _i32, _vp, _i32, _i64, _vp, _i32, _f32, _vp, _i64, _i32],
+    "psamd_state_space_prepare": [_vp, _vp, _vp, _vp, _vp, _i64, _i32],
+    "psamd_matrix_memory_gates": [_vp, _vp, _vp, _f32, _vp, _vp, _i64, _vp, _vp, _i32, _i32],
+    "psamd_matrix_memory_operands": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _vp, _vp, _i64],
+    "psamd_memory_read_norm_gate": [_vp, _vp, _vp, _i64, _i32, _i32, _f32, _vp, _f32, _vp, _i32, _i64, _vp, _i64],
+    "psamd_pool_kv_append": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
+    "psamd_attention_masked": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _i32,
+                               _vp, _vp, _vp, _i32, _vp],
 }
+
+ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2, "relu": 3}
 
 
 GATE_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
@@ -783,24 +799,151 @@ class HipOps:
 
     # ------------------------------------------------------------ delta rules
 
-    def short_conv(self, rows, col: int, conv_w, out, state, state_offset: int, ctx, silu: bool = True) -> None:
-        """out[t, c] = act(sum_j conv_w[c, j] v(t - (taps - 1) + j, c)), v = rows[:, col + c], over each item's
+    def short_conv(self, rows, col: int, conv_w, out, state, state_offset: int, ctx, silu: bool = True, bias=None) -> None:
+        """out[t, c] = act(bias[c] + sum_j conv_w[c, j] v(t - (taps - 1) + j, c)), v = rows[:, col + c], over each item's
         tokens, continued in front of an item's first token from the inputs its state slot saved
         (``state[slot, state_offset + j * channels + c]``, oldest first), which are then replaced by the
-        item's last taps - 1 inputs. ``out`` is float32 [T, channels]."""
+        item's last taps - 1 inputs. ``rows`` and ``out`` ([T, channels]) are float32 or bfloat16, each on its own;
+        ``bias`` is float32 [channels] or None."""
         t, channels = out.shape
         taps = conv_w.shape[1]
         self._need(rows.is_contiguous() and rows.shape[0] == t and 0 <= col and col + channels <= rows.shape[1], "short_conv: rows")
-        self._need(out.dtype == torch.float32 and out.is_contiguous() and conv_w.dtype == torch.float32
+        self._need(out.is_contiguous() and conv_w.dtype == torch.float32
                    and tuple(conv_w.shape) == (channels, taps) and conv_w.is_contiguous(), "short_conv: float32 taps [channels, taps] and output")
+        if bias is not None:
+            self._need(bias.dtype == torch.float32 and bias.numel() == channels and bias.is_contiguous(), "short_conv: the bias is float32 [channels]")
         self._need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
                    and 0 <= state_offset and state_offset + (taps - 1) * channels <= state.shape[1], "short_conv: the state's saved inputs")
         self._need(t == ctx.num_tokens, "short_conv: token count differs from the step batch")
-        self._ok(self.lib.psamd_short_conv(self._stream(), rows.data_ptr() + col * rows.element_size(), _code(rows.dtype),
-                                           rows.shape[1], conv_w.data_ptr(), out.data_ptr(), channels,
-                                           state.data_ptr() + 4 * state_offset, state.shape[1], ctx.tok_item.data_ptr(),
-                                           ctx.item_start.data_ptr(), ctx.slots.data_ptr(), t, ctx.num_items, channels, taps,
-                                           int(silu)))
+        self._ok(self.lib.psamd_short_conv_to(self._stream(), rows.data_ptr() + col * rows.element_size(), _code(rows.dtype),
+                                              rows.shape[1], conv_w.data_ptr(), _ptr(bias), out.data_ptr(), _code(out.dtype), channels,
+                                              state.data_ptr() + 4 * state_offset, state.shape[1], ctx.tok_item.data_ptr(),
+                                              ctx.item_start.data_ptr(), ctx.slots.data_ptr(), t, ctx.num_items, channels, taps,
+                                              int(silu)))
+
+    # ------------------------------------------ several streams, mixers side by side, recurrences through the delta scan
+
+    def stream_rms_norm(self, x, weight, eps: float) -> None:
+        """x (float32 [T, H]) <- weight * x / sqrt(mean(x^2) + eps), row by row and in place."""
+        t, h = x.shape
+        self._need(x.dtype == torch.float32 and x.is_contiguous() and weight.dtype == torch.float32 and weight.numel() == h
+                   and weight.is_contiguous(), "stream_rms_norm: float32 rows and weight")
+        self._ok(self.lib.psamd_stream_rms_norm(self._stream(), x.data_ptr(), weight.data_ptr(), float(eps), t, h))
+
+    def _streams(self, streams, what: str) -> tuple[int, int, int]:
+        self._need(streams.dtype == torch.float32 and streams.dim() == 3 and streams.is_contiguous() and 1 <= streams.shape[0] <= 16,
+                   f"{what}: the streams are float32 [count <= 16, T, H]")
+        return tuple(streams.shape)
+
+    def hyper_read(self, streams, read, weight, eps: float, out, factor=None) -> None:
+        """out = u / sqrt(mean(u^2) + eps) * weight (* factor), u = sum_s read[s] streams[s]; out [T, H] in its own dtype."""
+        count, t, h = self._streams(streams, "hyper_read")
+        for v, n in ((read, count), (weight, h)) + (((factor, h),) if factor is not None else ()):
+            self._need(v.dtype == torch.float32 and v.numel() == n and v.is_contiguous(), "hyper_read: float32 parameters")
+        self._need(out.shape == (t, h) and out.is_contiguous(), "hyper_read: output")
+        self._ok(self.lib.psamd_hyper_read(self._stream(), streams.data_ptr(), count, read.data_ptr(), weight.data_ptr(), float(eps),
+                                           _ptr(factor), out.data_ptr(), _code(out.dtype), t, h))
+
+    def hyper_write(self, streams, mix, write, delta) -> None:
+        """streams[t'] <- sum_s mix[s, t'] streams[s] + write[t'] delta, all copies at once from the old ones; delta is
+        [T, H] in a kernel dtype or [S, T, H] float32 slices."""
+        count, t, h = self._streams(streams, "hyper_write")
+        self._need(mix.dtype == torch.float32 and tuple(mix.shape) == (count, count) and mix.is_contiguous()
+                   and write.dtype == torch.float32 and write.numel() == count and write.is_contiguous(), "hyper_write: float32 parameters")
+        dptr, dcode, slices, stride = self._delta_args(delta, t, h, delta.dtype)
+        self._ok(self.lib.psamd_hyper_write(self._stream(), streams.data_ptr(), count, mix.data_ptr(), write.data_ptr(), dptr, dcode,
+                                            max(slices, 1), stride, t, h))
+
+    def weighted_sum(self, a, a_scale: float, b, b_scale: float, out) -> None:
+        """out (float32 [T, H]) = a_scale * a + b_scale * b; a and b are [T, H] in a kernel dtype or [S, T, H] float32 slices."""
+        t, h = out.shape
+        self._need(out.dtype == torch.float32 and out.is_contiguous(), "weighted_sum: the output is float32")
+        ap, ac, asl, ast = self._delta_args(a, t, h, a.dtype)
+        bp, bc, bsl, bst = self._delta_args(b, t, h, b.dtype)
+        self._ok(self.lib.psamd_weighted_sum(self._stream(), ap, ac, max(asl, 1), ast, float(a_scale), bp, bc, max(bsl, 1), bst,
+                                             float(b_scale), out.data_ptr(), t * h))
+
+    def activation(self, x, kind: str) -> None:
+        """x <- f(x) in place: "gelu" (exact), "gelu_tanh", "silu" or "relu"."""
+        self._need(x.is_contiguous(), "activation: a contiguous tensor")
+        self._ok(self.lib.psamd_activation(self._stream(), x.data_ptr(), _code(x.dtype), x.numel(), ACTIVATIONS[kind]))
+
+    def gated_group_norm(self, y, x, x_col: int, skip, heads: int, gate_rows, gate_col: int, weight, groups: int, eps: float, out) -> None:
+        """v = (y + skip[head] x) silu(gate); out = v / sqrt(mean(v^2) + eps) * weight over each of ``groups`` equal parts of
+        a row. y float32 [T, inner]; x float32 rows from column ``x_col``; the gate in ``gate_rows`` from ``gate_col``."""
+        t, inner = y.shape
+        self._need(y.dtype == torch.float32 and y.is_contiguous() and x.dtype == torch.float32 and x.is_contiguous()
+                   and x.shape[0] == t and 0 <= x_col and x_col + inner <= x.shape[1], "gated_group_norm: y and x are float32")
+        self._need(inner % heads == 0 and inner % groups == 0, "gated_group_norm: sizes")
+        for v, n in ((skip, heads), (weight, inner)):
+            self._need(v.dtype == torch.float32 and v.numel() == n and v.is_contiguous(), "gated_group_norm: float32 parameters")
+        self._need(gate_rows.is_contiguous() and gate_rows.shape[0] == t and 0 <= gate_col and gate_col + inner <= gate_rows.shape[1]
+                   and out.dtype == gate_rows.dtype and out.shape == (t, inner) and out.is_contiguous(), "gated_group_norm: gate and output")
+        self._ok(self.lib.psamd_gated_group_norm(self._stream(), y.data_ptr(), x.data_ptr() + 4 * x_col, x.shape[1], skip.data_ptr(), heads,
+                                                 gate_rows.data_ptr() + gate_col * gate_rows.element_size(), _code(gate_rows.dtype),
+                                                 gate_rows.shape[1], weight.data_ptr(), groups, float(eps), out.data_ptr(), t, inner))
+
+    def state_space_prepare(self, dt, dt_bias, decay_log, coef) -> None:
+        """dt float32 [T, heads] -> coef float32 [T, 3 heads] = [exp(-exp(decay_log) d) | 0 | d], d = softplus(dt + dt_bias)."""
+        t, heads = dt.shape
+        self._need(dt.dtype == torch.float32 and dt.is_contiguous() and coef.dtype == torch.float32 and coef.shape == (t, 3 * heads)
+                   and coef.is_contiguous(), "state_space_prepare: dt [T, heads] and coef [T, 3 heads] are float32")
+        for v in (dt_bias, decay_log):
+            self._need(v.dtype == torch.float32 and v.numel() == heads and v.is_contiguous(), "state_space_prepare: float32 [heads]")
+        self._ok(self.lib.psamd_state_space_prepare(self._stream(), dt.data_ptr(), dt_bias.data_ptr(), decay_log.data_ptr(),
+                                                    coef.data_ptr(), t, heads))
+
+    def matrix_memory_gates(self, gates, gate_bias, cap: float, coef, state, m_offset: int, ctx) -> None:
+        """gates float32 [T, 2 heads] = [input | forget] inputs; i = cap tanh((. + b) / cap), f = logsigmoid(cap tanh(.)); with
+        the running maximum m' = max(f + m, i) kept in ``state[slot, m_offset + h]``: coef float32 [T, 4 heads] =
+        [exp(f + m - m') | 0 | exp(i - m') | exp(-m')], token by token over each item."""
+        t = gates.shape[0]
+        heads = gates.shape[1] // 2
+        self._need(gates.dtype == torch.float32 and gates.is_contiguous() and coef.dtype == torch.float32
+                   and coef.shape == (t, 4 * heads) and coef.is_contiguous() and gate_bias.dtype == torch.float32
+                   and gate_bias.numel() == 2 * heads and gate_bias.is_contiguous(), "matrix_memory_gates: float32 operands")
+        self._need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous() and 0 <= m_offset
+                   and m_offset + heads <= state.shape[1] and t == ctx.num_tokens, "matrix_memory_gates: the state")
+        self._ok(self.lib.psamd_matrix_memory_gates(self._stream(), gates.data_ptr(), gate_bias.data_ptr(), float(cap), coef.data_ptr(),
+                                                    state.data_ptr() + 4 * m_offset, state.shape[1], ctx.item_start.data_ptr(),
+                                                    ctx.slots.data_ptr(), ctx.num_items, heads))
+
+    def matrix_memory_operands(self, rows, q_col: int, k_col: int, v_col: int, heads: int, dim: int, vdim: int, q_scale: float,
+                               u, vals) -> None:
+        """u float32 [T, 2 heads dim] = [q * q_scale | k]; vals float32 [T, heads (vdim + 1)] = per head [v | 1]."""
+        t = rows.shape[0]
+        self._need(rows.is_contiguous() and u.dtype == torch.float32 and u.shape == (t, 2 * heads * dim) and u.is_contiguous()
+                   and vals.dtype == torch.float32 and vals.shape == (t, heads * (vdim + 1)) and vals.is_contiguous(),
+                   "matrix_memory_operands: shapes")
+        self._ok(self.lib.psamd_matrix_memory_operands(self._stream(), rows.data_ptr(), _code(rows.dtype), rows.shape[1], q_col, k_col,
+                                                       v_col, heads, dim, vdim, float(q_scale), u.data_ptr(), vals.data_ptr(), t))
+
+    def memory_read_norm_gate(self, raw, coef, floor_col: int, heads: int, vdim: int, read_eps: float, weight, eps: float,
+                              gate_rows, gate_col: int, out) -> None:
+        """raw float32 [T, heads (vdim + 1)] = per head [S^T q | n . q]: o = S^T q / (max(|n . q|, coef[t, floor_col + h]) +
+        read_eps); out = o / sqrt(mean(o^2) + eps) * weight[h] * sigmoid(gate)."""
+        t = raw.shape[0]
+        self._need(raw.dtype == torch.float32 and raw.shape == (t, heads * (vdim + 1)) and raw.is_contiguous()
+                   and coef.dtype == torch.float32 and coef.is_contiguous() and coef.shape[0] == t and 0 <= floor_col
+                   and floor_col + heads <= coef.shape[1], "memory_read_norm_gate: raw and coef are float32")
+        self._need(weight.dtype == torch.float32 and weight.numel() == heads * vdim and weight.is_contiguous(), "memory_read_norm_gate: weight")
+        self._need(gate_rows.is_contiguous() and gate_rows.shape[0] == t and 0 <= gate_col and gate_col + heads * vdim <= gate_rows.shape[1]
+                   and out.dtype == gate_rows.dtype and out.shape == (t, heads * vdim) and out.is_contiguous(), "memory_read_norm_gate: gate and output")
+        self._ok(self.lib.psamd_memory_read_norm_gate(self._stream(), raw.data_ptr(), coef.data_ptr() + 4 * floor_col, coef.shape[1], heads,
+                                                      vdim, float(read_eps), weight.data_ptr(), float(eps),
+                                                      gate_rows.data_ptr() + gate_col * gate_rows.element_size(),
+                                                      _code(gate_rows.dtype), gate_rows.shape[1], out.data_ptr(), t))
+
+    def pool_kv_append(self, kv, pool_kv, ctx, group: int, pool_group: int, hkv: int, d: int, block: int) -> None:
+        """For every token of the step that completes a block of ``block`` tokens (the pool group's ``write_slot`` >= 0): the mean
+        of the block's keys and values as the token pages hold them goes to that place of the pool's pages."""
+        g, pg = ctx.groups[group], ctx.groups[pool_group]
+        for pages in (kv, pool_kv):
+            self._need(pages.shape[1:] == (2, hkv, 16 * d) and pages.is_contiguous() and pages.dtype == kv.dtype,
+                       "pool_kv_append: pages are [blocks, 2, kv_heads, 16*D] in one dtype")
+        self._ok(self.lib.psamd_pool_kv_append(self._stream(), kv.data_ptr(), pool_kv.data_ptr(), _code(kv.dtype), ctx.positions.data_ptr(),
+                                               ctx.tok_item.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(),
+                                               pg.write_slot.data_ptr(), ctx.num_tokens, hkv, d, block))
 
     def gated_delta_prepare(self, u, groups: int, dim: int, gates, decay_log, decay_bias, coef, q_scale: float,
                             unit_eps: float) -> None:
@@ -926,12 +1069,39 @@ class HipOps:
         return bool(self.lib.psamd_attention_mfma_supports(hq, hkv, d))
 
     def paged_attention(self, qkv, out, kv, ctx, group: int, hq: int, hkv: int, d: int, scale: float,
-                        window: int | None, exact_weights: bool = False, sink=None, dist_bias=None) -> None:
+                        window: int | None, exact_weights: bool = False, sink=None, dist_bias=None, keep_first: int = 0,
+                        pooled=None, head_gate=None) -> None:
         """``exact_weights``: the softmax weights enter the product with the values as computed in
         32-bit (the matrix-core kernels then take them as three bfloat16 terms that sum to the float32
         weight exactly) instead of rounded to bfloat16; the 32-bit kernels always do. ``sink``
         (float32 [hq]): exp(sink) joins every softmax's denominator. ``dist_bias`` (float32 [hq, n]):
-        entry [h, min(i - j, n - 1)] is added to the scaled score of query i and key j."""
+        entry [h, min(i - j, n - 1)] is added to the scaled score of query i and key j. ``keep_first``: the window also
+        sees the first that many positions. ``pooled`` = (pages, group, block): one mean key and value per block of tokens
+        wholly in front of the window, from pages of their own. ``head_gate`` (float32 [T, hq]): output times sigmoid."""
+        if keep_first or pooled is not None or head_gate is not None:
+            self._need(sink is None and dist_bias is None and window is not None and window >= 1,
+                       "attention: kept positions, pooled blocks and a gate per head go with a window and without sink or bias")
+            t = qkv.shape[0]
+            g = ctx.groups[group]
+            self._need(out.shape == (t, hq * d) and out.is_contiguous() and out.dtype == qkv.dtype and t == ctx.num_tokens, "attention: output")
+            self._need(kv.dtype == qkv.dtype and kv.shape[1:] == (2, hkv, 16 * d) and kv.is_contiguous(),
+                       "attention: cache must be [blocks, 2, kv_heads, 16*D] in the activation dtype")
+            pool_ptr = pool_off = pool_ids = None
+            block = 0
+            if pooled is not None:
+                pkv, pgroup, block = pooled
+                self._need(pkv.dtype == qkv.dtype and pkv.shape[1:] == (2, hkv, 16 * d) and pkv.is_contiguous() and block >= 1,
+                           "attention: the pooled blocks' pages")
+                pg = ctx.groups[pgroup]
+                pool_ptr, pool_off, pool_ids = pkv.data_ptr(), pg.table_off.data_ptr(), pg.block_ids.data_ptr()
+            if head_gate is not None:
+                self._need(head_gate.dtype == torch.float32 and head_gate.shape == (t, hq) and head_gate.is_contiguous(),
+                           "attention: the gate is float32 [T, hq]")
+            self._ok(self.lib.psamd_attention_masked(
+                self._stream(), qkv.data_ptr(), qkv.shape[1], out.data_ptr(), kv.data_ptr(), _code(qkv.dtype), t,
+                ctx.positions.data_ptr(), ctx.tok_item.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d,
+                float(scale), int(window), int(keep_first), pool_ptr, pool_off, pool_ids, int(block), _ptr(head_gate)))
+            return
         if sink is not None:
             self._need(sink.dtype == torch.float32 and sink.numel() == hq and sink.is_contiguous(), "attention: sink is float32 [hq]")
         if dist_bias is not None:

@@ -26,6 +26,8 @@ class LayerCache:
     kv: torch.Tensor
     group: int
     window: int | None
+    # Further entries of the same run by the mixer's own names (``Mixer.aux_cache_needs``).
+    aux: "dict[str, LayerCache] | None" = None
 
 
 def slot_size(head_dim: int, value_dim: int, largest: int = 256) -> int:
@@ -106,14 +108,26 @@ class PagedAttention(Mixer):
       row bucket(i - j) is added to the scaled score of query i and key j (``distance_bucket``).
     * ``head_scale``: a learned number per query head (name "head_scale") that multiplies the head's
       scores beside ``scale``. It is folded, in 32-bit, into the factor each query head is multiplied
-      with behind its norm (a weight per head instead of one shared by the heads)."""
+      with behind its norm (a weight per head instead of one shared by the heads).
+    * ``keep_first`` (with ``window``): a query also sees the sequence's first that many positions,
+      at their true places, however far back they lie; their pages are never given back.
+    * ``pooled_block`` = P (with ``window``): beside the window's tokens a query at position i sees one
+      key and one value for every block of P tokens that lies wholly in front of its window
+      (block b = positions bP .. bP + P - 1, seen once bP + P - 1 <= i - window): the means of the
+      block's keys and values as the pages hold them, in the same softmax. The means live in a
+      cache entry of their own with one place per P tokens (``aux_cache_needs``: "pool"), written
+      when the block's last token runs; tokens that have left the window and whose block is not
+      complete in front of it are not seen.
+    * ``head_gate``: a number per query head and token, sigmoid(W x)_h (name "head_gate",
+      [heads, hidden]), multiplies the head's output before the output matrix; 32-bit."""
 
     def __init__(self, hidden_size: int, positions: Mapping[str, PositionEncoding], num_heads: int,
                  num_kv_heads: int, head_dim: int, names: Mapping[str, str], position: str | None = None,
                  window: int | None = None, scale: float | None = None, value_dim: int | None = None,
                  qk_norm_eps: float | None = None, own_kv: bool = True, exact_weights: bool = False,
                  qk_bias: bool = False, qk_norm_weights: bool = False, values_are_keys: bool = False,
-                 sink: bool = False, distance_bias: Mapping[str, Any] | None = None, head_scale: bool = False) -> None:
+                 sink: bool = False, distance_bias: Mapping[str, Any] | None = None, head_scale: bool = False,
+                 keep_first: int = 0, pooled_block: int = 0, head_gate: bool = False) -> None:
         if num_kv_heads < 1 or num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads not divisible by {num_kv_heads} kv heads")
         self.hidden_size = int(hidden_size)
@@ -125,6 +139,11 @@ class PagedAttention(Mixer):
         self.qk_bias, self.qk_norm_weights = bool(qk_bias), bool(qk_norm_weights)
         self.values_are_keys, self.has_sink = bool(values_are_keys), bool(sink)
         self.head_scale = bool(head_scale)
+        self.keep_first, self.pooled_block, self.head_gate = int(keep_first), int(pooled_block), bool(head_gate)
+        if (self.keep_first or self.pooled_block) and window is None:
+            raise ValueError("kept first positions and pooled blocks belong to a sliding window")
+        if self.keep_first < 0 or self.pooled_block < 0 or (self.pooled_block and not own_kv):
+            raise ValueError("bad kept positions or pooled block (pooled blocks need keys of the layer's own)")
         self.distance_bias = None if distance_bias is None else (int(distance_bias["buckets"]), float(distance_bias["far"]))
         if self.qk_norm_weights and self.qk_norm_eps is None:
             raise ValueError("weights on the q/k norm need qk_norm_eps")
@@ -135,7 +154,11 @@ class PagedAttention(Mixer):
         if self.distance_bias is not None and not 2 <= self.distance_bias[0] < 2 * self.distance_bias[1]:
             raise ValueError(f"a distance bias needs at least 2 buckets and a reach beyond half of them, got {self.distance_bias}")
         extras = (self.qk_bias or self.qk_norm_weights or self.values_are_keys or self.has_sink
-                  or self.distance_bias is not None or self.head_scale)
+                  or self.distance_bias is not None or self.head_scale or self.keep_first or self.pooled_block
+                  or self.head_gate)
+        self.masked = bool(self.keep_first or self.pooled_block or self.head_gate)
+        if self.masked and (self.has_sink or self.distance_bias is not None):
+            raise ValueError("kept positions, pooled blocks and a gate per head are not combined with a sink or a distance bias")
         self.bias = self.q_norm_weight = self.k_norm_weight = self.sink = self.distance_table = None
         self.names = dict(names)
         self.window = None if window is None else int(window)
@@ -185,10 +208,20 @@ class PagedAttention(Mixer):
             want[n["sink"]] = WeightWant((self.num_heads,), "bias")
         if self.distance_bias is not None:
             want[n["rel"]] = WeightWant((self.distance_bias[0], self.num_heads), "bias")
+        if self.head_gate:
+            want[n["head_gate"]] = WeightWant((self.num_heads, h))
         return want
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(self.num_kv_heads, self.slots, self.window)
+        if self.pooled_block:
+            # A block's tokens must still be in their pages when its last one runs.
+            return CacheNeed(self.num_kv_heads, self.slots, max(self.window, self.pooled_block), self.keep_first)
+        return CacheNeed(self.num_kv_heads, self.slots, self.window, self.keep_first)
+
+    def aux_cache_needs(self) -> dict[str, CacheNeed]:
+        if not self.pooled_block:
+            return {}
+        return {"pool": CacheNeed(self.num_kv_heads, self.slots, None, 0, self.pooled_block)}
 
     def _spread(self, w: torch.Tensor, heads: int, size: int, index: "list[int] | None") -> torch.Tensor:
         """Rows [heads * size, K] laid into [heads * slots, K]; ``index``: slot of each row of a head."""
@@ -239,13 +272,16 @@ class PagedAttention(Mixer):
                 self._spread(torch.ones((self.head_dim, 1)), 1, self.head_dim, self.index).view(-1)
             self.q_norm_weight = on_device((per_head * shared[None, :]).reshape(-1))
             self.q_weight_per_head = True
+        if self.head_gate:
+            self.w_gate = rt.ops.prepare_matrix(tensors[n["head_gate"]], rt)
         if self.has_sink:
             self.sink = on_device(tensors[n["sink"]])
         if self.distance_bias is not None:
             self.distance_table = on_device(distance_table(tensors[n["rel"]].to(torch.float32), self.distance_bias[1]))
 
     def weight_bytes(self) -> int:
-        return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o))
+        gate = self.w_gate.numel() * self.w_gate.element_size() if self.head_gate else 0
+        return sum(w.numel() * w.element_size() for w in (self.w_qkv, self.w_o)) + gate
 
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: Any, state: torch.Tensor | None,
                 writes_cache: bool) -> torch.Tensor:
@@ -282,7 +318,21 @@ class PagedAttention(Mixer):
                                         cache.kv if writes_cache else None, ctx.groups[cache.group].write_slot,
                                         norm_dim, eps)
         out = ws.get("attn.out", (t, self.q_size), rt.dtype)
-        if self.sink is not None or self.distance_table is not None:
+        if self.masked:
+            gate = pooled = None
+            if self.head_gate:
+                gate = ws.get("attn.gate", (t, self.num_heads), torch.float32)
+                ops.linear(x, self.w_gate, gate)
+            if self.pooled_block:
+                pool = cache.aux["pool"]
+                if writes_cache:
+                    ops.pool_kv_append(cache.kv, pool.kv, ctx, cache.group, pool.group, self.num_kv_heads, self.slots,
+                                       self.pooled_block)
+                pooled = (pool.kv, pool.group, self.pooled_block)
+            ops.paged_attention(qkv, out, cache.kv, ctx, cache.group, self.num_heads, self.num_kv_heads,
+                                self.slots, self.scale, self.window, exact_weights=self.exact_weights,
+                                keep_first=self.keep_first, pooled=pooled, head_gate=gate)
+        elif self.sink is not None or self.distance_table is not None:
             ops.paged_attention(qkv, out, cache.kv, ctx, cache.group, self.num_heads, self.num_kv_heads,
                                 self.slots, self.scale, cache.window, exact_weights=self.exact_weights,
                                 sink=self.sink, dist_bias=self.distance_table)

@@ -35,11 +35,16 @@ class WeightWant:
 class CacheNeed:
     """Keys and values in pages. Layers whose needs are equal share a page pool and a
     block table per request ("layer group"); ``window`` None keeps every key, a number
-    keeps only the last ``window`` positions and lets older pages go."""
+    keeps only the last ``window`` positions and lets older pages go, except those that hold
+    one of the first ``keep_first`` positions. ``stride`` n: the entry holds one key and value
+    per n tokens (entry b once token b n + n - 1 has run), so a request of L tokens has
+    L // n entries in it and a page covers 16 n tokens."""
 
     kv_heads: int
     head_dim: int
     window: int | None = None
+    keep_first: int = 0
+    stride: int = 1
 
 
 @dataclass(frozen=True)
@@ -198,6 +203,16 @@ class Mixer(Part):
 
     def state_need(self) -> StateNeed | None:
         return None
+
+    def aux_cache_needs(self) -> "dict[str, CacheNeed]":
+        """Further cache entries beside the one ``cache_need`` describes (means over blocks of
+        tokens, say), by a name of the mixer's choosing: the run's ``LayerCache.aux[name]``."""
+        return {}
+
+    # Where in a slot's row this mixer's state begins. 0 when the mixer is the only owner of the
+    # run's state; a container (a block with state of its own, a mixer made of several) lays its
+    # parts' states side by side and sets this before the first step.
+    state_base = 0
 
     # True: ``forward`` takes ``NormedRows`` for x (it hands x to kernels that normalize their
     # tokens themselves); the block then lets the norm in front of it be lazy.

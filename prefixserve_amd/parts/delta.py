@@ -98,7 +98,7 @@ class GatedDeltaRule(Mixer):
         gates = ws.get("delta.gates", (t, 2 * hd), torch.float32)                         # [strength logits | decay inputs]
         ops.linear(x, self.w_coef, gates)
         u = ws.get("delta.u", (t, self.channels), torch.float32)
-        ops.short_conv(rows, 0, self.conv_w, u, state, 0, ctx, silu=True)
+        ops.short_conv(rows, 0, self.conv_w, u, state, self.state_base, ctx, silu=True)
         coef = ws.get("delta.coef", (t, 3 * hd), torch.float32)                           # [g | -b | b]
         ops.gated_delta_prepare(u, self.num_kv_heads, self.head_dim, gates, self.decay_log, self.decay_bias, coef,
                                 self.head_dim ** -0.5, UNIT_EPS)
@@ -106,7 +106,7 @@ class GatedDeltaRule(Mixer):
         k_col, v_col = self.key_size, 2 * self.key_size
         ops.delta_scan(keys=(u, k_col), directions=(u, k_col), removals=(u, k_col), queries=(u, 0),
                        key_groups=self.num_kv_heads, decay_vectors=None, decay=(coef, 0), removal_scale=(coef, hd),
-                       value_scale=(coef, 2 * hd), values=(u, v_col), out=o, state=state, state_offset=self.tail, ctx=ctx,
+                       value_scale=(coef, 2 * hd), values=(u, v_col), out=o, state=state, state_offset=self.state_base + self.tail, ctx=ctx,
                        heads=hd, dim=self.head_dim, vdim=self.value_dim, reads_decayed=True)
         out = ws.get("delta.out", (t, self.value_size), rt.dtype)
         ops.heads_norm_gate(o, hd, self.value_dim, self.norm_w, False, self.norm_eps, rows, self.channels, "silu", out)
@@ -178,7 +178,7 @@ class GeneralizedDeltaRule(Mixer):
         o = ws.get("gdelta.o", (t, s), torch.float32)
         ops.delta_scan(keys=(operands, s), directions=(operands, 5 * s), removals=(operands, 4 * s), queries=(operands, 0),
                        key_groups=hd, decay_vectors=(operands, 3 * s), decay=None, removal_scale=None, value_scale=None,
-                       values=(operands, 2 * s), out=o, state=state, state_offset=0, ctx=ctx, heads=hd, dim=self.head_dim,
+                       values=(operands, 2 * s), out=o, state=state, state_offset=self.state_base, ctx=ctx, heads=hd, dim=self.head_dim,
                        vdim=self.head_dim, reads_decayed=False)
         out = ws.get("gdelta.out", (t, s), rt.dtype)
         ops.heads_norm_gate(o, hd, self.head_dim, self.norm_w, True, self.norm_eps, rows, 3 * s, "sigmoid", out)

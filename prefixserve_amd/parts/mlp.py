@@ -54,4 +54,36 @@ class SwiGLU(FeedForward):
         return ops.linear_to_residual(act, self.w_down, "mlp.delta", getattr(ctx, "residual", None))
 
 
+class DenseMLP(FeedForward):
+    """down( act(up(x)) ), no gate and no biases. ``activation``: "gelu" (the exact one, with erf),
+    "gelu_tanh", "silu" or "relu". ``names``: "up", "down"."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, names: Mapping[str, str], activation: str = "gelu") -> None:
+        if activation not in ("gelu", "gelu_tanh", "silu", "relu"):
+            raise ValueError(f"the feed-forward's activation {activation!r} is not implemented")
+        self.activation = activation
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.names = dict(names)
+
+    def weights(self) -> dict[str, WeightWant]:
+        h, i, n = self.hidden_size, self.intermediate_size, self.names
+        return {n["up"]: WeightWant((i, h)), n["down"]: WeightWant((h, i))}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        super().bind(tensors, rt)
+        self.w_up = rt.ops.prepare_matrix(tensors[self.names["up"]], rt)
+        self.w_down = rt.ops.prepare_matrix(tensors[self.names["down"]], rt)
+
+    def weight_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_up, self.w_down))
+
+    def forward(self, x: torch.Tensor, ctx: "StepContext") -> torch.Tensor:
+        rt, ops, ws = self.rt, self.rt.ops, self.rt.workspace
+        act = ws.get("mlp.act", (x.shape[0], self.intermediate_size), rt.dtype)
+        ops.linear(x, self.w_up, act)
+        ops.activation(act, self.activation)
+        return ops.linear_to_residual(act, self.w_down, "mlp.delta", getattr(ctx, "residual", None))
+
+
 register_feed_forward("swiglu", SwiGLU)
+register_feed_forward("dense_mlp", DenseMLP)

@@ -11,12 +11,15 @@ import torch
 from . import attention as _attention  # noqa: F401  (registers the built-in parts)
 from . import block as _block  # noqa: F401
 from . import delta as _delta  # noqa: F401
+from . import hyper as _hyper  # noqa: F401
 from . import latent as _latent  # noqa: F401
 from . import mlp as _mlp  # noqa: F401
 from . import moe as _moe  # noqa: F401
 from . import norm as _norm  # noqa: F401
+from . import parallel as _parallel  # noqa: F401
 from . import recurrent as _recurrent  # noqa: F401
 from . import rope as _rope  # noqa: F401
+from . import ssm as _ssm  # noqa: F401
 from . import stream as _stream  # noqa: F401
 from .base import CacheNeed, Part, Runtime, StateNeed, WeightWant, make
 from .spec import ModelSpec
@@ -115,24 +118,50 @@ class DecoderModel:
                 continue
             if run.writes_cache:
                 needs[run.cache] = need
+        # A mixer's further entries get numbers of their own behind every run's.
+        for key, need in self._aux_entries().items():
+            needs[self._aux_ids[key]] = need
         return needs
+
+    def _aux_entries(self) -> dict[tuple[int, str], CacheNeed]:
+        """(cache entry of the writing run, the mixer's name for it) -> need, and their entry numbers."""
+        out: dict[tuple[int, str], CacheNeed] = {}
+        for run in self.spec.order:
+            if run.writes_cache:
+                for name, need in self.blocks[run.layer].mixer.aux_cache_needs().items():
+                    out[(run.cache, name)] = need
+        base = 1 + max((run.cache for run in self.spec.order), default=0)
+        self._aux_ids = {key: base + i for i, key in enumerate(sorted(out))}
+        return out
 
     def state_needs(self) -> dict[int, StateNeed]:
         """index into ``spec.order`` -> fixed-size per-request state its mixer keeps."""
         needs: dict[int, StateNeed] = {}
         for i, run in enumerate(self.spec.order):
-            need = self.blocks[run.layer].mixer.state_need()
+            need = self._block_state_need(self.blocks[run.layer])
             if need is not None:
                 needs[i] = need
         return needs
 
+    @staticmethod
+    def _block_state_need(blk: Any) -> StateNeed | None:
+        """A block may keep state of its own around its mixer's (``state_need`` of the block);
+        otherwise the run's state is the mixer's."""
+        own = getattr(blk, "state_need", None)
+        return own() if own is not None else blk.mixer.state_need()
+
     def state_in_graphs(self) -> bool:
-        """Whether every mixer that keeps state lets a captured decode step update it."""
-        return all(blk.mixer.state_in_graphs for blk in self.blocks if blk.mixer.state_need() is not None)
+        """Whether every part that keeps state lets a captured decode step update it."""
+        return all(getattr(blk, "state_in_graphs", blk.mixer.state_in_graphs) for blk in self.blocks
+                   if self._block_state_need(blk) is not None)
 
     def attach(self, caches: Mapping[int, Any], states: Mapping[int, torch.Tensor]) -> None:
         self.caches = dict(caches)
         self.states = dict(states)
+        for (entry, name), _need in self._aux_entries().items():
+            main, aux = self.caches.get(entry), self.caches.get(self._aux_ids[(entry, name)])
+            if main is not None and aux is not None:
+                main.aux = {**(main.aux or {}), name: aux}
 
     # ------------------------------------------------------------------- step
 
@@ -146,10 +175,17 @@ class DecoderModel:
         s, ws, ops = self.spec, rt.workspace, rt.ops
         t = ctx.num_tokens
         with ops.step_scope():
-            residual = ws.get("residual", (t, s.hidden_size), torch.float32)
+            if s.streams > 1:
+                # Every copy of the stream starts as the token table's output; blocks get all of them.
+                streams = ws.get("residual", (s.streams, t, s.hidden_size), torch.float32)
+                residual = streams[0]
+            else:
+                streams = residual = ws.get("residual", (t, s.hidden_size), torch.float32)
             ops.embed(ctx.token_ids, self.embedding, residual)
             for tr in self.embedding_transforms:
                 tr.apply(residual, ctx, None)
+            if s.streams > 1:
+                streams[1:].copy_(residual.unsqueeze(0).expand(s.streams - 1, t, s.hidden_size))
             ctx.residual = residual
             ctx.stream_copy = None           # a context may be stepped twice (a graph's eager run, then its capture)
             if self.keeps_embedding_output:
@@ -167,10 +203,14 @@ class DecoderModel:
                     ctx.pass_index = run.pass_index
                     for name in run.before:
                         self.stream_transforms[name].apply(residual, ctx, None)
-                pending = self.blocks[run.layer].forward(residual, pending, ctx, self.caches.get(run.cache),
+                pending = self.blocks[run.layer].forward(streams, pending, ctx, self.caches.get(run.cache),
                                                          self.states.get(i), run.writes_cache)
             if ctx.num_logit_rows == 0:
                 return None
+            if s.streams > 1:
+                # The final norm reads the sum of the copies: the others join the first as slices to be added.
+                assert pending is None, "a block over several streams leaves nothing pending"
+                pending = streams[1:]
             x = self.final_norm.add_norm_rows(residual, pending, ctx.logit_rows, "final.x", lazy=True)
             logits = ws.get("logits", (ctx.num_logit_rows, s.vocab_size), torch.float32)
             ops.linear(x, self.head, logits)

@@ -14,20 +14,26 @@ class RMSNorm(Norm):
     residual sum in 32-bit (prefixserve/model/llama.py:63-69 of the reference upcasts the
     same way). The weight is used in the dtype it is stored in. ``unit_offset``: the stored
     tensor is the weight's distance from one, the factor is 1 + w (formed in 32-bit and kept so:
-    rounding 1 + w to the stored 16 bits would drop most of w)."""
+    rounding 1 + w to the stored 16 bits would drop most of w). ``scalar``: the stored weight is one
+    number for all coordinates (a tensor without dimensions); it is spread over the width at bind
+    time, in 32-bit."""
 
-    def __init__(self, hidden_size: int, eps: float, name: str = "weight", unit_offset: bool = False) -> None:
+    def __init__(self, hidden_size: int, eps: float, name: str = "weight", unit_offset: bool = False,
+                 scalar: bool = False) -> None:
         self.hidden_size = int(hidden_size)
         self.eps = float(eps)
         self.name = name
         self.unit_offset = bool(unit_offset)
+        self.scalar = bool(scalar)
 
     def weights(self) -> dict[str, WeightWant]:
-        return {self.name: WeightWant((self.hidden_size,), "offset" if self.unit_offset else "norm")}
+        return {self.name: WeightWant(() if self.scalar else (self.hidden_size,), "offset" if self.unit_offset else "norm")}
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
         super().bind(tensors, rt)
         w = tensors[self.name]
+        if self.scalar:
+            w = w.to(torch.float32).reshape(1).expand(self.hidden_size)
         if w.dtype not in (torch.bfloat16, torch.float32):
             w = w.to(torch.float32)
         if self.unit_offset:

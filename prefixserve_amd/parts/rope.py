@@ -11,6 +11,10 @@ from .base import RotaryTable, Runtime, register_position
 
 
 def rope_inv_freq(head_dim: int, theta: float, scaling: Mapping[str, Any] | None) -> torch.Tensor:
+    return rope_inv_freq64(head_dim, theta, scaling).to(torch.float32)
+
+
+def rope_inv_freq64(head_dim: int, theta: float, scaling: Mapping[str, Any] | None) -> torch.Tensor:
     """inv_freq[i] = 1 / theta^(2i/D), i < D/2, then the llama3 three bands by wavelength:
     long waves divided by ``factor``, short ones unchanged, the middle blended
     (prefixserve/model/llama.py:24-46 of the reference). Evaluated in float64 and rounded
@@ -30,7 +34,7 @@ def rope_inv_freq(head_dim: int, theta: float, scaling: Mapping[str, Any] | None
         smoothed = (1.0 - smooth) * scaled / factor + smooth * scaled
         medium = ~(wavelen < high_wavelen) & ~(wavelen > low_wavelen)
         inv = torch.where(medium, smoothed, scaled)
-    return inv.to(torch.float32)
+    return inv
 
 
 class RotaryEmbedding(RotaryTable):
@@ -38,11 +42,20 @@ class RotaryEmbedding(RotaryTable):
     (prefixserve/model/llama.py:72-77). The angle is a float32 product as in the
     reference's table (llama.py:56-58); its cosine and sine are kept in float32 whatever
     the activation dtype. The table is ``[max_position, D/2, 2]`` = (cos, sin) and is
-    read by the kernel that also writes keys and values into their pages."""
+    read by the kernel that also writes keys and values into their pages.
 
-    def __init__(self, head_dim: int, theta: float, scaling: Mapping[str, Any] | None = None) -> None:
+    ``rotary_dim``: only the model's first that many dimensions of a head rotate (partners
+    rotary_dim / 2 apart, frequencies theta^(-2i / rotary_dim)); the table's other pair slots are the
+    identity and the mixer lays a head out accordingly. The angles of this form are products in
+    float64, rounded once as cosine and sine."""
+
+    def __init__(self, head_dim: int, theta: float, scaling: Mapping[str, Any] | None = None,
+                 rotary_dim: int | None = None) -> None:
         if head_dim % 2:
             raise ValueError(f"rotary head_dim must be even, got {head_dim}")
+        if rotary_dim is not None and (rotary_dim % 2 or not 0 <= rotary_dim <= head_dim):
+            raise ValueError(f"rotary_dim {rotary_dim} must be even and at most head_dim {head_dim}")
+        self.rotary_dim = None if rotary_dim is None else int(rotary_dim)
         self.head_dim = int(head_dim)
         self.theta = float(theta)
         self.scaling = dict(scaling) if scaling is not None else None
@@ -52,6 +65,17 @@ class RotaryEmbedding(RotaryTable):
         super().bind(tensors, rt)
 
     def prepare(self, max_position: int) -> None:
+        if self.rotary_dim is not None:
+            table = torch.zeros((max_position, self.head_dim // 2, 2), dtype=torch.float64)
+            table[:, :, 0] = 1.0
+            if self.rotary_dim:
+                inv = rope_inv_freq64(self.rotary_dim, self.theta, self.scaling)
+                angle = torch.outer(torch.arange(max_position, dtype=torch.float64), inv)
+                table[:, : self.rotary_dim // 2, 0] = angle.cos()
+                table[:, : self.rotary_dim // 2, 1] = angle.sin()
+            self.table = table.to(torch.float32).contiguous().to(self.rt.device)
+            self.max_position = int(max_position)
+            return
         inv = rope_inv_freq(self.head_dim, self.theta, self.scaling)
         pos = torch.arange(max_position, dtype=torch.float32)
         angle = torch.outer(pos, inv)  # float32 product, exactly rounded

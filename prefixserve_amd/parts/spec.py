@@ -81,9 +81,15 @@ class ModelSpec:
     # Named transforms of the residual stream between layers (a re-entry into a repeated stretch,
     # say), applied where a ``LayerRun.before`` names them; each is built once.
     stream_transforms: Mapping[str, PartSpec] = field(default_factory=dict)
+    # Copies of the residual stream. With more than one the stream is [streams, T, hidden]: every
+    # copy starts as the token table's output (behind its transforms), the layers' blocks read and
+    # write all of them, and the final norm reads their sum.
+    streams: int = 1
 
     def validate(self) -> None:
         writers: dict[int, int] = {}
+        if self.streams < 1:
+            raise ValueError(f"{self.streams} residual streams")
         for run in self.order:
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"order names layer {run.layer}, model has {len(self.layers)}")

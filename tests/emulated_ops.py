@@ -42,7 +42,7 @@ class EmulatedOps:
     def add_rmsnorm_rows(self, residual, delta, rows, weight, eps, out) -> None:
         x = residual[rows.long()]
         if delta is not None:
-            x = x + delta[rows.long()].float()
+            x = x + (delta[:, rows.long()].float().sum(0) if delta.dim() == 3 else delta[rows.long()].float())
         out.copy_((weight.float() * x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)).to(out.dtype))
 
     def linear(self, x, w, out) -> None:
@@ -253,7 +253,7 @@ class EmulatedOps:
         ang = positions.double()[:, None] * freq[torch.arange(h) // 2][None, :]
         x.add_(torch.where(torch.arange(h) % 2 == 0, torch.sin(ang), torch.cos(ang)).float())
 
-    def short_conv(self, rows, col, conv_w, out, state, state_offset, ctx, silu=True) -> None:
+    def short_conv(self, rows, col, conv_w, out, state, state_offset, ctx, silu=True, bias=None) -> None:
         channels, taps = conv_w.shape
         keep = taps - 1
         starts = ctx.item_start.tolist()
@@ -261,10 +261,10 @@ class EmulatedOps:
             t0, t1 = starts[i], starts[i + 1]
             saved = state[int(ctx.slots[i]), state_offset: state_offset + keep * channels].view(keep, channels)
             v = torch.cat([saved, rows[t0:t1, col: col + channels].float()], dim=0)
-            acc = torch.zeros((t1 - t0, channels))
+            acc = torch.zeros((t1 - t0, channels)) if bias is None else bias.expand(t1 - t0, channels).clone()
             for j in range(taps):
                 acc += conv_w[:, j] * v[j: j + t1 - t0]
-            out[t0:t1] = torch.nn.functional.silu(acc) if silu else acc
+            out[t0:t1] = (torch.nn.functional.silu(acc) if silu else acc).to(out.dtype)
             if keep:
                 saved.copy_(v[-keep:].clone())
 
@@ -328,8 +328,121 @@ class EmulatedOps:
         """[keys, kv_heads, d] -> [keys, heads, d]: query head h reads kv head h // rep."""
         return x.repeat_interleave(rep, dim=1)
 
+    # ----------------------------------------------- several streams, side-by-side mixers, dense feed-forward
+
+    def stream_rms_norm(self, x, weight, eps) -> None:
+        x.copy_(weight * x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps))
+
+    def hyper_read(self, streams, read, weight, eps, out, factor=None) -> None:
+        u = torch.einsum("s,sth->th", read, streams)
+        h = weight.float() * u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps)
+        out.copy_((h if factor is None else h * factor).to(out.dtype))
+
+    def hyper_write(self, streams, mix, write, delta) -> None:
+        y = delta.float().sum(0) if delta.dim() == 3 else delta.float()
+        streams.copy_(torch.einsum("st,sxh->txh", mix, streams) + write[:, None, None] * y[None])
+
+    def weighted_sum(self, a, a_scale, b, b_scale, out) -> None:
+        def whole(d):
+            return d.float().sum(0) if d.dim() == 3 else d.float()
+        out.copy_(a_scale * whole(a) + b_scale * whole(b))
+
+    def activation(self, x, kind) -> None:
+        f = {"gelu": torch.nn.functional.gelu, "gelu_tanh": lambda z: torch.nn.functional.gelu(z, approximate="tanh"),
+             "silu": torch.nn.functional.silu, "relu": torch.relu}[kind]
+        x.copy_(f(x.float()).to(x.dtype))
+
+    def gated_group_norm(self, y, x, x_col, skip, heads, gate_rows, gate_col, weight, groups, eps, out) -> None:
+        t, inner = y.shape
+        v = y + (skip[:, None] * x[:, x_col: x_col + inner].view(t, heads, inner // heads)).reshape(t, inner)
+        g = v * torch.nn.functional.silu(gate_rows[:, gate_col: gate_col + inner].float())
+        g = g.view(t, groups, inner // groups)
+        g = g * torch.rsqrt((g * g).mean(-1, keepdim=True) + eps)
+        out.copy_((g.reshape(t, inner) * weight).to(out.dtype))
+
+    def state_space_prepare(self, dt, dt_bias, decay_log, coef) -> None:
+        d = torch.nn.functional.softplus(dt + dt_bias)
+        coef.copy_(torch.cat([torch.exp(-torch.exp(decay_log) * d), torch.zeros_like(d), d], dim=-1))
+
+    def matrix_memory_gates(self, gates, gate_bias, cap, coef, state, m_offset, ctx) -> None:
+        heads = gates.shape[1] // 2
+        starts = ctx.item_start.tolist()
+        for i in range(ctx.num_items):
+            m = state[int(ctx.slots[i]), m_offset: m_offset + heads]
+            for t in range(starts[i], starts[i + 1]):
+                z = cap * torch.tanh((gates[t] + gate_bias) / cap)
+                il, fl = z[:heads], torch.nn.functional.logsigmoid(z[heads:])
+                m_new = torch.maximum(fl + m, il)
+                coef[t] = torch.cat([torch.exp(fl + m - m_new), torch.zeros(heads), torch.exp(il - m_new), torch.exp(-m_new)])
+                m.copy_(m_new)
+
+    def matrix_memory_operands(self, rows, q_col, k_col, v_col, heads, dim, vdim, q_scale, u, vals) -> None:
+        t = rows.shape[0]
+        u[:, : heads * dim] = rows[:, q_col: q_col + heads * dim].float() * q_scale
+        u[:, heads * dim:] = rows[:, k_col: k_col + heads * dim].float()
+        v = vals.view(t, heads, vdim + 1)
+        v[:, :, :vdim] = rows[:, v_col: v_col + heads * vdim].float().view(t, heads, vdim)
+        v[:, :, vdim] = 1.0
+
+    def memory_read_norm_gate(self, raw, coef, floor_col, heads, vdim, read_eps, weight, eps, gate_rows, gate_col, out) -> None:
+        t = raw.shape[0]
+        r = raw.view(t, heads, vdim + 1)
+        den = torch.maximum(r[:, :, vdim].abs(), coef[:, floor_col: floor_col + heads]) + read_eps
+        o = r[:, :, :vdim] / den[:, :, None]
+        o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * weight.view(heads, vdim)
+        z = gate_rows[:, gate_col: gate_col + heads * vdim].float().view(t, heads, vdim)
+        out.copy_((o * torch.sigmoid(z)).reshape(t, heads * vdim).to(out.dtype))
+
+    def pool_kv_append(self, kv, pool_kv, ctx, group, pool_group, hkv, d, block) -> None:
+        g, pg = ctx.groups[group], ctx.groups[pool_group]
+        offs = g.table_off.tolist()
+        for t in range(ctx.num_tokens):
+            slot = int(pg.write_slot[t])
+            if slot < 0:
+                continue
+            pos, item = int(ctx.positions[t]), int(ctx.tok_item[t])
+            ks, vs = [], []
+            for j in range(pos - block + 1, pos + 1):
+                page = int(g.block_ids[offs[item] + j // PAGE])
+                ks.append(kv[page, 0].view(hkv, PAGE, d)[:, j % PAGE].float())
+                vs.append(kv[page, 1].view(hkv, d, PAGE)[:, :, j % PAGE].float())
+            pool_kv[slot // PAGE, 0].view(hkv, PAGE, d)[:, slot % PAGE] = torch.stack(ks).mean(0).to(kv.dtype)
+            pool_kv[slot // PAGE, 1].view(hkv, d, PAGE)[:, :, slot % PAGE] = torch.stack(vs).mean(0).to(kv.dtype)
+
+    def _masked_attention(self, qkv, out, kv, ctx, group, hq, hkv, d, scale, window, keep_first, pooled, head_gate) -> None:
+        g = ctx.groups[group]
+        t = qkv.shape[0]
+        rep = hq // hkv
+        offs = g.table_off.tolist()
+        for row in range(t):
+            pos, item = int(ctx.positions[row]), int(ctx.tok_item[row])
+            seen = [j for j in range(pos + 1) if pos - j < window or j < keep_first]
+            keys, vals = [], []
+            for j in seen:
+                page = int(g.block_ids[offs[item] + j // PAGE])
+                keys.append(kv[page, 0].view(hkv, PAGE, d)[:, j % PAGE].float())
+                vals.append(kv[page, 1].view(hkv, d, PAGE)[:, :, j % PAGE].float())
+            if pooled is not None:
+                pkv, pgroup, block = pooled
+                pg = ctx.groups[pgroup]
+                poffs = pg.table_off.tolist()
+                for b in range(max(0, (pos - window + 1) // block)):
+                    page = int(pg.block_ids[poffs[item] + b // PAGE])
+                    keys.append(pkv[page, 0].view(hkv, PAGE, d)[:, b % PAGE].float())
+                    vals.append(pkv[page, 1].view(hkv, d, PAGE)[:, :, b % PAGE].float())
+            keys = torch.stack(keys).repeat_interleave(rep, dim=1)          # [n, hq, d]
+            vals = torch.stack(vals).repeat_interleave(rep, dim=1)
+            q = qkv[row, : hq * d].view(hq, d).float()
+            w = torch.softmax(torch.einsum("hd,nhd->hn", q, keys) * scale, dim=-1)
+            o = torch.einsum("hn,nhd->hd", w, vals)
+            if head_gate is not None:
+                o = o * torch.sigmoid(head_gate[row])[:, None]
+            out[row] = o.reshape(hq * d).to(out.dtype)
+
     def paged_attention(self, qkv, out, kv, ctx, group, hq, hkv, d, scale, window, exact_weights=False, sink=None,
-                        dist_bias=None) -> None:
+                        dist_bias=None, keep_first=0, pooled=None, head_gate=None) -> None:
+        if keep_first or pooled is not None or head_gate is not None:
+            return self._masked_attention(qkv, out, kv, ctx, group, hq, hkv, d, scale, window, keep_first, pooled, head_gate)
         g = ctx.groups[group]
         t = qkv.shape[0]
         q = qkv[:, : hq * d].view(t, hq, d).float()
