@@ -193,10 +193,6 @@ def _mixer(kind: str, m: Mapping[str, Any], where: str) -> Any:
         return StateSpace.from_json(m, where)
     _only(m, ("left", "right", "left_scale", "right_scale"), where)
     left = WindowAttention.from_json(m["left"], where + ".left")
-    if kind == "parallel" and (left.rot is not None or left.pool):
-        raise UnsupportedModelError(f"{where}.left: a 'parallel' layer's attention has no rotation and no pooled blocks")
-    if kind == "parallel_2" and left.keep_first:
-        raise UnsupportedModelError(f"{where}.left: a 'parallel_2' layer's attention keeps no first tokens")
     return SideBySide(left, RIGHT[kind].from_json(m["right"], where + ".right"), float(m.get("left_scale", 1.0)),
                       float(m.get("right_scale", 1.0)))
 
