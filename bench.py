@@ -157,8 +157,46 @@ def larupel_pair(size: dict, layers: int, vocab: int) -> tuple[dict, dict]:
     return larupel, llama
 
 
+# Fubelorn at sizes that resemble real layers, beside the Llama decoder of equal size: same width, the attention's head
+# counts and head size, the same inner feed-forward size. Four layers over four residual streams, four taps in front of
+# every sub-layer: a state space layer (inner size 2 x width, state 128), attention in a window of 1,024 with blocks of 64
+# pooled in front of it beside a matrix memory, and twice attention in a window of 1,024 that keeps four first tokens
+# beside a gated delta rule.
+FUBELORN_SIZES = {
+    "fubelorn-w2048-h32x64-ff8192": dict(width=2048, heads=32, kv_heads=8, dim=64, ff=8192, ssm_heads=64, ssm_dim=64, state=128,
+                                         memory_heads=8, memory_dim=128, delta_heads=16, delta_kv=8, delta_dim=128),
+    "fubelorn-w4096-h32x128-ff14336": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=14336, ssm_heads=64, ssm_dim=128, state=128,
+                                           memory_heads=16, memory_dim=128, delta_heads=32, delta_kv=16, delta_dim=128),
+}
+
+
+def fubelorn_pair(size: dict, layers: int, vocab: int) -> tuple[dict, dict]:
+    """(Fubelorn config.json, the Llama config.json of equal size). ``layers`` is not used: the pattern has four."""
+    ff = {"kind": "dense", "ff": size["ff"]}
+    att = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"], "scale": size["dim"] ** -0.5}
+    kept = dict(att, mask={"size": 1024, "keep_first": 4})
+    pooled = dict(att, mask={"size": 1024, "pool": 64},
+                  rot={"dims": size["dim"], "base": 500000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}})
+    delta = {"heads": size["delta_heads"], "kv_heads": size["delta_kv"], "dim": size["delta_dim"], "vdim": size["delta_dim"], "conv": 4}
+    memory = {"heads": size["memory_heads"], "dim": size["memory_dim"], "vdim": size["memory_dim"], "gate_cap": 15.0}
+    side = lambda left, right: {"left": left, "right": right, "left_scale": 1.0, "right_scale": 0.5}
+    entries = [
+        {"type": "mamba2", "mlp": ff, "mixer": {"heads": size["ssm_heads"], "vdim": size["ssm_dim"], "state": size["state"], "groups": 1,
+                                                "conv": 4, "norm_groups": 1}},
+        {"type": "parallel_2", "mlp": ff, "mixer": side(pooled, memory)},
+        {"type": "parallel", "mlp": ff, "mixer": side(kept, delta)},
+        {"type": "parallel", "mlp": ff, "mixer": side(kept, delta)},
+    ]
+    fubelorn = {"architecture": "Fubelorn", "vocab": vocab, "width": size["width"], "norm": {"eps": 1e-6}, "residual_mult": 0.3,
+                "streams": 4, "canon": {"taps": 4}, "layers": entries}
+    llama = dict(LLAMA_1B, vocab_size=vocab, hidden_size=size["width"], intermediate_size=size["ff"], num_hidden_layers=4,
+                 num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                 tie_word_embeddings=False)
+    return fubelorn, llama
+
+
 def compare_designs(args) -> int:
-    """Prefill and decode throughput of another design's layers (Radivik, Gokolix, Larupel) beside Llama layers of
+    """Prefill and decode throughput of another design's layers (Radivik, Gokolix, Larupel, Fubelorn) beside Llama layers of
     equal size, through the same runner and step function. One JSON line; the default benchmark is not run."""
     import numpy as np
     import torch
@@ -170,7 +208,10 @@ def compare_designs(args) -> int:
     rng = np.random.default_rng(0)
     vocab, layers = 32000, args.layers or 4
     prompt, batch, context = args.prompt_len, args.batch, args.context
-    if args.compare in LARUPEL_SIZES or args.compare == "larupel":
+    if args.compare in FUBELORN_SIZES or args.compare == "fubelorn":
+        design, pair_of = "fubelorn", fubelorn_pair
+        sizes = FUBELORN_SIZES if args.compare == "fubelorn" else {args.compare: FUBELORN_SIZES[args.compare]}
+    elif args.compare in LARUPEL_SIZES or args.compare == "larupel":
         design, pair_of = "larupel", larupel_pair
         sizes = LARUPEL_SIZES if args.compare == "larupel" else {args.compare: LARUPEL_SIZES[args.compare]}
     elif args.compare in GOKOLIX_SIZES or args.compare == "gokolix":
@@ -289,12 +330,12 @@ def main() -> int:
     ap.add_argument("--no-peaks", action="store_true", help="skip measuring the copy bandwidth and a large library product")
     ap.add_argument("--model", default=None, help="use this model folder instead of writing random weights")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="llama-3.2-1b", help="layer sizes of the random model")
-    ap.add_argument("--compare", choices=sorted(RADIVIK_SIZES) + ["all"] + sorted(GOKOLIX_SIZES) + ["gokolix"] + sorted(LARUPEL_SIZES) + ["larupel"],
-                    default=None,
-                    help="instead of the benchmark: Radivik, Gokolix or Larupel layers of this size ('all': every Radivik size, "
-                         "'gokolix' / 'larupel': every size of that design) beside Llama layers of equal size (prefill of --prompt-len tokens, "
+    ap.add_argument("--compare", choices=sorted(RADIVIK_SIZES) + ["all"] + sorted(GOKOLIX_SIZES) + ["gokolix"] + sorted(LARUPEL_SIZES) + ["larupel"]
+                    + sorted(FUBELORN_SIZES) + ["fubelorn"], default=None,
+                    help="instead of the benchmark: Radivik, Gokolix, Larupel or Fubelorn layers of this size ('all': every Radivik size, "
+                         "'gokolix' / 'larupel' / 'fubelorn': every size of that design) beside Llama layers of equal size (prefill of --prompt-len tokens, "
                          "decoding at --batch in --context; --layers, default 4, for Radivik)")
-    ap.add_argument("--compare-only", choices=["both", "radivik", "gokolix", "larupel", "llama"], default="both")
+    ap.add_argument("--compare-only", choices=["both", "radivik", "gokolix", "larupel", "fubelorn", "llama"], default="both")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

@@ -364,7 +364,7 @@ def test_long_contexts_windows_and_blocks_of_real_sizes(dtype, tmp_path):
     for i, key in ((0, "keep_first"), (2, "pool")):
         other = json.loads(json.dumps(raw))
         other["layers"][i]["mixer"]["left"]["mask"][key] = 0
-        assert rel(plain.forward(other, tensors, toks)[-1], truth[-1]) > 100 * F32_TOL
+        assert rel(plain.forward(other, tensors, toks)[-1], truth[-1]) > 50 * F32_TOL
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
