@@ -377,6 +377,299 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
   }
 }
 
+// ------------------------------------------------------------------ a window with more to see than the window
+
+// The per-head kernel above for a sliding window whose queries also see the sequence's first keep_first
+// positions and, with pool != NULL, one mean key and value per block of `block` tokens that lies wholly
+// in front of their window (block b for the query at position i once b * block + block - 1 <= i - window),
+// read from pages of their own through a table of their own. The keys are numbered in tiles of 32 in three
+// runs (kept positions in front of the first window tile, the window's tiles, the blocks), which the four
+// waves take in turn; everything else is the kernel above with one run of keys per tile of queries.
+// Single tokens run as tiles of one query (dec_items). `gate` (float [tokens, hq] or NULL): the head's
+// output times sigmoid(gate[t, h]).
+template <int NS, bool P3 = false>
+__global__ __launch_bounds__(256) void attn_masked_mfma_kernel(
+    const bf16_t* __restrict__ qkv, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ kv,
+    const int32_t* __restrict__ pf_tiles, const int32_t* __restrict__ dec_items, const int32_t* __restrict__ item_start,
+    const int32_t* __restrict__ item_pos0, const int32_t* __restrict__ table_off,
+    const int32_t* __restrict__ block_ids, int hq, int hkv, float scale, int window, int keep_first,
+    const bf16_t* __restrict__ pool, const int32_t* __restrict__ pool_table_off,
+    const int32_t* __restrict__ pool_block_ids, int block, const float* __restrict__ gate) {
+  float* part_o = nullptr;
+  float* part_ml = nullptr;
+  const Extras ex = {nullptr, nullptr, 0};
+  constexpr int D = 16 * NS;
+  constexpr int DT = (D + 31) / 32;
+  constexpr int DTC = DT < 2 ? DT : 2;      // d-tiles merged per pass (bounds the LDS buffer)
+  __shared__ float sm_m[4][32], sm_l[4][32];
+  __shared__ float sm_o[3 * DTC * 16 * 64];
+  extern __shared__ int32_t table[];
+  // Late tiles of a prompt see the most keys: start them first. Workgroups are handed out in
+  // the order x + gridDim.x * y, round robin over the dies: x runs over the kv heads first and
+  // then over the query heads of each, so that with a multiple of 8 kv heads all workgroups of
+  // a kv head run on one die and share its keys and values in that die's L2.
+  const int tile = gridDim.y - 1 - blockIdx.y;
+  const int h = (blockIdx.x % hkv) * (hq / hkv) + blockIdx.x / hkv;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // The tiles of the step's portions, or (dec_items) one tile for each of its single tokens.
+  const int item = dec_items != nullptr ? dec_items[tile] : pf_tiles[2 * tile];
+  const int q_off = dec_items != nullptr ? 0 : pf_tiles[2 * tile + 1];
+  const int t0 = item_start[item];
+  const int n = item_start[item + 1] - t0;
+  const int pos0 = item_pos0[item];
+  const int kvh = h / (hq / hkv);
+  const int col = lane & 31, hi = lane >> 5;
+
+  const int qi = min(q_off + col, n - 1);          // lanes past the end repeat the last query
+  const bool q_valid = q_off + col < n;
+  const int q_pos = pos0 + qi;
+  const int first_pos = pos0 + q_off;
+  const int last_pos = pos0 + min(q_off + 31, n - 1);
+  const int max_key = pos0 + n - 1;
+  const int k_lo_q = window > 0 ? max(0, q_pos - window + 1) : 0;
+  const int k_begin_vis = window > 0 ? max(0, first_pos - window + 1) : 0;   // the first key any query of the tile sees
+  const int k_begin = k_begin_vis & ~31;
+  const float c = scale * 1.44269504088896340736f;  // scores are exponentiated in base 2
+  const int nsplit = 1;                 // one run of keys per tile of queries
+  const int64_t part_slot = 0;
+  // The keys a query sees, numbered in tiles of 32: the kept first positions in front of the first
+  // window tile, the window's tiles, the pooled blocks wholly in front of some query's window.
+  const int n_keep = min(keep_first, k_begin);
+  const int u_win = (n_keep + 31) & ~31;
+  const int n_win = ((last_pos - k_begin) / 32 + 1) * 32;
+  const int nb_max = pool != nullptr ? max(0, (last_pos - window + 1) / block) : 0;
+  const int nb_q = pool != nullptr ? max(0, (q_pos - window + 1) / block) : 0;
+  const int u_pool = u_win + n_win;
+  const int u_end = u_pool + ((nb_max + 31) & ~31);
+  const int token_pages = (last_pos >> 4) + 1;
+  int32_t* ptable = table + token_pages;
+  {
+    const int32_t* gtable = block_ids + table_off[item];
+    for (int i = threadIdx.x; i < token_pages; i += blockDim.x) table[i] = gtable[i];
+    if (nb_max > 0) {
+      const int32_t* gp = pool_block_ids + pool_table_off[item];
+      for (int i = threadIdx.x; i <= ((nb_max - 1) >> 4); i += blockDim.x) ptable[i] = gp[i];
+    }
+  }
+  __syncthreads();
+
+  bf16x8 qf[NS];
+  {
+    const bf16_t* qp = qkv + static_cast<int64_t>(t0 + qi) * q_stride + h * D + 8 * hi;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) qf[s] = ld8(qp + 16 * s);
+  }
+
+  f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[dt][v] = 0.f;
+  float m = -INFINITY, l = 0.f;       // m in base-2 units (score * c)
+
+  const int64_t page_elems = 2LL * hkv * kPage * D;
+  const int64_t khead = static_cast<int64_t>(kvh) * kPage * D;
+  const int64_t vhead = static_cast<int64_t>(hkv) * kPage * D + static_cast<int64_t>(kvh) * D * kPage;
+
+  struct Tile {
+    bf16x8 k[NS];        // A operand of S^T = K.Q^T: key row (k0 + col), 8 dims per 16-wide step
+    bf16x8 v[2][DT];     // A operand of O^T += V^T.P^T: page c of the tile, V^T row d
+  };
+  auto load_tile = [&](Tile& t, int u) {
+    const bool pooled = u >= u_pool && nb_max > 0;   // a tile past the end (loaded ahead, never used) reads window keys
+    const int k0 = pooled ? u - u_pool : u >= u_win ? k_begin + (u - u_win) : u;
+    const int last_key = pooled ? max(nb_max - 1, 0) : last_pos;
+    const bf16_t* src = pooled ? pool : kv;
+    const int32_t* tab = pooled ? ptable : table;
+    const int key_a = min(k0 + col, last_key);
+    const bf16_t* kp = src + static_cast<int64_t>(tab[key_a >> 4]) * page_elems + khead + (key_a & 15) * D + 8 * hi;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) t.k[i] = ld8(kp + 16 * i);
+#pragma unroll
+    for (int cpage = 0; cpage < 2; ++cpage) {
+      const int key_p = min(k0 + 16 * cpage, last_key);
+      const bf16_t* vp = src + static_cast<int64_t>(tab[key_p >> 4]) * page_elems + vhead + 4 * hi;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const bf16_t* vr = vp + min(32 * dt + col, D - 1) * kPage;
+        t.v[cpage][dt] = join(ld4(vr), ld4(vr + 8));
+      }
+    }
+    // Values in places nobody of this request has written are set to zero (see zero_unless).
+    const int lo = pooled || u < u_win ? 0 : k_begin_vis;
+    const int top = pooled ? nb_max - 1 : u < u_win ? n_keep - 1 : max_key;
+    if (k0 + 31 > top || k0 < lo) {
+#pragma unroll
+      for (int cpage = 0; cpage < 2; ++cpage)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          t.v[cpage][dt] = zero_unless(t.v[cpage][dt], [&](int e) {
+            const int key = k0 + 16 * cpage + 8 * (e >> 2) + 4 * hi + (e & 3);
+            return key <= top && (key >= lo || key < keep_first);
+          });
+    }
+  };
+  auto compute = [&](const Tile& t, int u) {
+    const bool pooled = u >= u_pool && nb_max > 0;   // a tile past the end (loaded ahead, never used) reads window keys
+    const int k0 = pooled ? u - u_pool : u >= u_win ? k_begin + (u - u_win) : u;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    f32x16 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.k[0], qf[0], zero, 0, 0, 0);
+#pragma unroll
+    for (int i = 1; i < NS; ++i) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.k[i], qf[i], s, 0, 0, 0);
+    if (ex.bias != nullptr) {
+      // The bias is added to the scaled score: here the score is still unscaled.
+      const float* bt = ex.bias + static_cast<int64_t>(h) * ex.n_dist;
+      const float unscale = 1.f / scale;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = k0 + 8 * (v >> 2) + 4 * hi + (v & 3);
+        s[v] = fmaf(bt[min(max(q_pos - key, 0), ex.n_dist - 1)], unscale, s[v]);
+      }
+    }
+    // Kept positions in front of every window: all of them. Window tiles: up to the query, from its
+    // window's first key on or kept. Pooled blocks: those wholly in front of the query's window.
+    {
+      const int top = pooled ? nb_q - 1 : u < u_win ? n_keep - 1 : q_pos;
+      const int lo = pooled || u < u_win ? 0 : k_lo_q;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = k0 + 8 * (v >> 2) + 4 * hi + (v & 3);
+        s[v] = (key <= top && (key >= lo || key < keep_first)) ? s[v] : -INFINITY;
+      }
+    }
+    float mx = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave)) * c;
+    // The running maximum is only raised (and the accumulators rescaled) when some query's
+    // scores outgrow it by more than 2^8: probabilities stay below 256, nothing overflows,
+    // the final division by the sum is exact either way, and most tiles skip the rescale of
+    // the whole accumulator.
+    if (__any(mx > m + 8.f)) {
+      const float m_new = fmaxf(m, mx);
+      const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[dt][v] *= alpha;
+      m = m_new;
+    }
+    const float m_use = m == -INFINITY ? 0.f : m;
+    float rowsum = 0.f;
+    bf16x8 pb[2], pm[2], pl[2];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[v], c, -m_use));
+      rowsum += p;
+      const WeightTerms w = split_weight<P3>(p);
+      pb[v >> 3][v & 7] = w.hi;
+      pm[v >> 3][v & 7] = w.mid;
+      pl[v >> 3][v & 7] = w.lo;
+    }
+    l += rowsum + __shfl_xor(rowsum, 32, kWave);
+#pragma unroll
+    for (int cpage = 0; cpage < 2; ++cpage)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.v[cpage][dt], pb[cpage], o[dt], 0, 0, 0);
+        if (P3) {
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.v[cpage][dt], pm[cpage], o[dt], 0, 0, 0);
+          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(t.v[cpage][dt], pl[cpage], o[dt], 0, 0, 0);
+        }
+      }
+  };
+
+  {
+    Tile ta, tb;
+    int k0 = 32 * wave;                   // a number of the tile list above, not a position
+    const int k_last = u_end - 1;
+    if (k0 <= k_last) {
+      load_tile(ta, k0);
+      while (true) {
+        // The next tile is loaded whether or not it exists (addresses are clamped to the last
+        // key): with no branch around the loads, the wait in front of the matrix instructions
+        // counts exactly the loads of the current tile and leaves the next tile's in flight.
+        load_tile(tb, k0 + 128);
+        compute(ta, k0);
+        k0 += 128;
+        if (k0 > k_last) break;
+        load_tile(ta, k0 + 128);
+        compute(tb, k0);
+        k0 += 128;
+        if (k0 > k_last) break;
+      }
+    }
+  }
+
+  // ---- merge the 4 waves' partial results for the 32 queries
+  if (hi == 0) {
+    sm_m[wave][col] = m;
+    sm_l[wave][col] = l;
+  }
+  __syncthreads();
+  float mm = sm_m[0][col];
+#pragma unroll
+  for (int w = 1; w < 4; ++w) mm = fmaxf(mm, sm_m[w][col]);
+  float ll = 0.f, mine = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float mw = sm_m[w][col];
+    const float f = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - mm);
+    ll += f * sm_l[w][col];
+    if (w == wave) mine = f;
+  }
+  // One run of several: the sum, the maximum and the output as it is go to the merge kernel.
+  if (nsplit == 1 && ex.sink != nullptr) ll += __builtin_amdgcn_exp2f(ex.sink[h] * kLog2e - mm);   // one run: the sink joins here
+  float inv = 1.f / ll;
+  if (gate != nullptr) inv *= 1.f / (1.f + __expf(-gate[static_cast<int64_t>(t0 + qi) * hq + h]));
+  if (nsplit > 1 && wave == 0 && q_valid && hi == 0) {
+    part_ml[2 * part_slot] = mm;
+    part_ml[2 * part_slot + 1] = ll;
+  }
+  bf16_t* op = out + static_cast<int64_t>(t0 + qi) * (static_cast<int64_t>(hq) * D) + h * D;
+#pragma unroll
+  for (int d0 = 0; d0 < DT; d0 += DTC) {
+    if (wave > 0) {
+#pragma unroll
+      for (int dt = 0; dt < DTC; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (d0 + dt < DT) sm_o[(((wave - 1) * DTC + dt) * 16 + v) * 64 + lane] = o[d0 + dt][v] * mine;
+    }
+    __syncthreads();
+    if (wave == 0 && q_valid) {
+#pragma unroll
+      for (int dt = 0; dt < DTC; ++dt) {
+        if (d0 + dt >= DT) continue;
+        float r[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          r[v] = o[d0 + dt][v] * mine;
+#pragma unroll
+          for (int w = 0; w < 3; ++w) r[v] += sm_o[((w * DTC + dt) * 16 + v) * 64 + lane];
+        }
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {
+          const int d = 32 * (d0 + dt) + 8 * v4 + 4 * hi;
+          if (d < D && nsplit > 1) {
+            *reinterpret_cast<float4*>(part_o + part_slot * D + d) =
+                float4{r[4 * v4 + 0], r[4 * v4 + 1], r[4 * v4 + 2], r[4 * v4 + 3]};
+          } else if (d < D) {
+            ushort4 pk;
+            pk.x = float_to_bf16(r[4 * v4 + 0] * inv);
+            pk.y = float_to_bf16(r[4 * v4 + 1] * inv);
+            pk.z = float_to_bf16(r[4 * v4 + 2] * inv);
+            pk.w = float_to_bf16(r[4 * v4 + 3] * inv);
+            *reinterpret_cast<ushort4*>(op + d) = pk;
+          }
+        }
+      }
+    }
+    if (d0 + DTC < DT) __syncthreads();
+  }
+}
+
 // ------------------------------------------------------------------ prefill, query heads of a kv head together
 
 // The same 32 queries for up to 4 query heads that share a kv head: one head per wave, all
@@ -1377,6 +1670,62 @@ int psamd_attention_prefill(void* stream, const void* qkv, int q_stride, void* o
     default: PSAMD_PF(16);
   }
 #undef PSAMD_PF
+}
+
+// Attention in a window that also sees the first keep_first positions and, with pool != NULL, the means over
+// blocks of `block` tokens wholly in front of the window (see attn_masked_mfma_kernel): the step's portions as
+// tiles of 32 queries (pf_tiles) and its single tokens as tiles of one (dec_items), in two launches.
+// max_kv_len sizes the two block tables staged in LDS.
+int psamd_attention_masked_mfma(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
+                                const int32_t* pf_tiles, int n_tiles, const int32_t* dec_items, int n_dec, int max_kv_len,
+                                const int32_t* item_start, const int32_t* item_pos0, const int32_t* table_off,
+                                const int32_t* block_ids, int hq, int hkv, int head_dim, float scale, int window,
+                                int keep_first, const void* pool, const int32_t* pool_table_off,
+                                const int32_t* pool_block_ids, int block, const float* gate, int exact_weights) {
+  PSAMD_REQUIRE(psamd_attention_mfma_supports(hq, hkv, head_dim), "shape not supported by the matrix-core kernels");
+  PSAMD_REQUIRE(q_stride % 8 == 0, "query row stride must be a multiple of 8 elements");
+  PSAMD_REQUIRE(max_kv_len >= 1 && max_kv_len <= 4096 * kPage, "context too long for the block tables staged in LDS");
+  PSAMD_REQUIRE(window >= 1 && keep_first >= 0, "kept first positions and pooled blocks belong to a window");
+  PSAMD_REQUIRE(pool == nullptr || (block >= 1 && pool_table_off != nullptr && pool_block_ids != nullptr),
+                "pooled blocks need their size and their pages' tables");
+  PSAMD_REQUIRE(n_tiles >= 0 && n_tiles <= 65535 && n_dec >= 0 && n_dec <= 65535, "too many query tiles for one launch");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t pages = static_cast<size_t>(ceil_div(max_kv_len, kPage)) + 1 +
+                       (pool != nullptr ? static_cast<size_t>(ceil_div(ceil_div(max_kv_len, block), kPage)) + 1 : 0);
+  const size_t smem = sizeof(int32_t) * pages;
+#define PSAMD_MASKED_LAUNCH(NS_, P3_, TILES_, DEC_, COUNT_)                                                          \
+  if ((COUNT_) > 0) {                                                                                                \
+    attn_masked_mfma_kernel<NS_, P3_><<<dim3(hq, (COUNT_)), dim3(256), smem, s>>>(                                   \
+        static_cast<const bf16_t*>(qkv), q_stride, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(kv), TILES_, \
+        DEC_, item_start, item_pos0, table_off, block_ids, hq, hkv, scale, window, keep_first,                      \
+        static_cast<const bf16_t*>(pool), pool_table_off, pool_block_ids, block, gate);                             \
+    const int rc = check_launch("psamd_attention_masked_mfma");                                                      \
+    if (rc != 0) return rc;                                                                                          \
+  }
+#define PSAMD_MASKED(NS_)                                                     \
+  {                                                                           \
+    if (exact_weights) {                                                      \
+      PSAMD_MASKED_LAUNCH(NS_, true, pf_tiles, nullptr, n_tiles)              \
+      PSAMD_MASKED_LAUNCH(NS_, true, nullptr, dec_items, n_dec)               \
+    } else {                                                                  \
+      PSAMD_MASKED_LAUNCH(NS_, false, pf_tiles, nullptr, n_tiles)             \
+      PSAMD_MASKED_LAUNCH(NS_, false, nullptr, dec_items, n_dec)              \
+    }                                                                         \
+    return 0;                                                                 \
+  }
+  switch (head_dim / 16) {
+    case 1: PSAMD_MASKED(1)
+    case 2: PSAMD_MASKED(2)
+    case 3: PSAMD_MASKED(3)
+    case 4: PSAMD_MASKED(4)
+    case 5: PSAMD_MASKED(5)
+    case 6: PSAMD_MASKED(6)
+    case 7: PSAMD_MASKED(7)
+    case 8: PSAMD_MASKED(8)
+    default: return fail("psamd_attention_masked_mfma: head sizes up to 128 (psamd_attention_masked takes the others)");
+  }
+#undef PSAMD_MASKED
+#undef PSAMD_MASKED_LAUNCH
 }
 
 // Whether the single-token items of a step have one context far longer than the rest: more than

@@ -114,6 +114,8 @@ _SIGNATURES = {
     "psamd_matrix_memory_operands": [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _vp, _vp, _i64],
     "psamd_memory_read_norm_gate": [_vp, _vp, _vp, _i64, _i32, _i32, _f32, _vp, _f32, _vp, _i32, _i64, _vp, _i64],
     "psamd_pool_kv_append": [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32],
+    "psamd_attention_masked_mfma": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
+                                    _f32, _i32, _i32, _vp, _vp, _vp, _i32, _vp, _i32],
     "psamd_attention_masked": [_vp, _vp, _i32, _vp, _vp, _i32, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _i32,
                                _vp, _vp, _vp, _i32, _vp],
 }
@@ -1097,6 +1099,16 @@ class HipOps:
             if head_gate is not None:
                 self._need(head_gate.dtype == torch.float32 and head_gate.shape == (t, hq) and head_gate.is_contiguous(),
                            "attention: the gate is float32 [T, hq]")
+            if (qkv.dtype == torch.bfloat16 and qkv.shape[1] % 8 == 0 and d <= 128 and self.mfma_attention_supported(hq, hkv, d)
+                    and self.MFMA_ATTENTION_EXTRAS and (self.fixed_kv_len or ctx.max_kv_len) <= 65536):
+                # The matrix cores: portions as tiles of 32 queries, single tokens as tiles of one.
+                kv_len = self.fixed_kv_len or ctx.max_kv_len
+                self._ok(self.lib.psamd_attention_masked_mfma(
+                    self._stream(), qkv.data_ptr(), qkv.shape[1], out.data_ptr(), kv.data_ptr(), ctx.pf_tiles.data_ptr(),
+                    ctx.num_prefill_tiles, ctx.dec_items.data_ptr(), ctx.num_decode, kv_len, ctx.item_start.data_ptr(),
+                    ctx.item_pos0.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d, float(scale),
+                    int(window), int(keep_first), pool_ptr, pool_off, pool_ids, int(block), _ptr(head_gate), int(exact_weights)))
+                return
             self._ok(self.lib.psamd_attention_masked(
                 self._stream(), qkv.data_ptr(), qkv.shape[1], out.data_ptr(), kv.data_ptr(), _code(qkv.dtype), t,
                 ctx.positions.data_ptr(), ctx.tok_item.data_ptr(), g.table_off.data_ptr(), g.block_ids.data_ptr(), hq, hkv, d,
