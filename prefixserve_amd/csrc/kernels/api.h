@@ -196,10 +196,11 @@ int psamd_stream_rms_norm(void* stream, float* x, const float* weight, float eps
 // [count, tokens, hidden], out in out_dtype.
 int psamd_hyper_read(void* stream, const float* streams, int count, const float* read, const float* weight, float eps,
                      const float* factor, void* out, int out_dtype, int64_t tokens, int hidden);
-// streams[t', t, :] <- sum_s mix[s, t'] streams[s, t, :] + write[t'] y[t, :], every copy from the old ones; y is one
-// tensor in delta_dtype or `slices` float slices.
-int psamd_hyper_write(void* stream, float* streams, int count, const float* mix, const float* write, const void* delta,
-                      int delta_dtype, int slices, int64_t slice_stride, int64_t tokens, int hidden);
+// streams[t', t, :] <- sum_s mix[s, t'] streams[s, t, :] + write[t'] y[t, :], every copy from the old ones; y = a_scale a
+// (+ b_scale b, b may be NULL), each one tensor in its dtype or float slices a stride apart.
+int psamd_hyper_write(void* stream, float* streams, int count, const float* mix, const float* write, const void* a,
+                      int a_dtype, int a_slices, int64_t a_stride, float a_scale, const void* b, int b_dtype, int b_slices,
+                      int64_t b_stride, float b_scale, int64_t tokens, int hidden);
 // out = a_scale * a + b_scale * b (float, n entries); a and b as the delta of psamd_hyper_write.
 int psamd_weighted_sum(void* stream, const void* a, int a_dtype, int a_slices, int64_t a_stride, float a_scale, const void* b,
                        int b_dtype, int b_slices, int64_t b_stride, float b_scale, float* out, int64_t n);

@@ -66,22 +66,27 @@ __global__ __launch_bounds__(256) void hyper_read_kernel(const float* __restrict
   }
 }
 
-// One thread per (token, channel): new[t] = sum_s mix[s, t] old[s] + write[t] * y, y = the delta (one
-// tensor in delta_dtype, or `slices` float slices slice_stride apart, added in ascending order).
+__device__ __forceinline__ float delta_at(const void* d, int dtype, int slices, int64_t stride, int64_t e) {
+  if (slices > 1 || dtype == kF32) {
+    const float* f = static_cast<const float*>(d);
+    float y = f[e];
+    for (int s = 1; s < slices; ++s) y += f[s * stride + e];
+    return y;
+  }
+  return bf16_to_float(static_cast<const bf16_t*>(d)[e]);
+}
+
+// One thread per (token, channel): new[t] = sum_s mix[s, t] old[s] + write[t] * y, y = a_scale * a (+ b_scale * b): each
+// one tensor in its dtype, or float slices a stride apart, added in ascending order.
 __global__ __launch_bounds__(256) void hyper_write_kernel(float* __restrict__ streams, int64_t stream_stride, int count,
                                                           const float* __restrict__ mix, const float* __restrict__ write,
-                                                          const void* __restrict__ delta, int delta_dtype, int slices,
-                                                          int64_t slice_stride, int64_t n) {
+                                                          const void* __restrict__ a, int a_dtype, int a_slices, int64_t a_stride,
+                                                          float a_scale, const void* __restrict__ b, int b_dtype, int b_slices,
+                                                          int64_t b_stride, float b_scale, int64_t n) {
   const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (e >= n) return;
-  float y;
-  if (slices > 1 || delta_dtype == kF32) {
-    const float* d = static_cast<const float*>(delta);
-    y = d[e];
-    for (int s = 1; s < slices; ++s) y += d[s * slice_stride + e];
-  } else {
-    y = bf16_to_float(static_cast<const bf16_t*>(delta)[e]);
-  }
+  float y = a_scale * delta_at(a, a_dtype, a_slices, a_stride, e);
+  if (b != nullptr) y = fmaf(b_scale, delta_at(b, b_dtype, b_slices, b_stride, e), y);
   float old[kMaxStreams];
 #pragma unroll
   for (int s = 0; s < kMaxStreams; ++s) old[s] = s < count ? streams[s * stream_stride + e] : 0.f;
@@ -95,16 +100,6 @@ __global__ __launch_bounds__(256) void hyper_write_kernel(float* __restrict__ st
       streams[t * stream_stride + e] = v;
     }
   }
-}
-
-__device__ __forceinline__ float delta_at(const void* d, int dtype, int slices, int64_t stride, int64_t e) {
-  if (slices > 1 || dtype == kF32) {
-    const float* f = static_cast<const float*>(d);
-    float y = f[e];
-    for (int s = 1; s < slices; ++s) y += f[s * stride + e];
-    return y;
-  }
-  return bf16_to_float(static_cast<const bf16_t*>(d)[e]);
 }
 
 __global__ __launch_bounds__(256) void weighted_sum_kernel(const void* __restrict__ a, int a_dtype, int a_slices, int64_t a_stride,
@@ -174,32 +169,48 @@ __global__ __launch_bounds__(256) void state_space_prepare_kernel(const float* _
   c[2 * heads + h] = d;
 }
 
-// grid (items), threads over heads: the gates of a matrix memory with their running maximum m, token by
-// token. gates row = [input | forget] inputs (heads each); i = cap tanh((. + b) / cap), f = logsigmoid(cap tanh(.));
+// grid (items, heads), one wave: the gates of a matrix memory with their running maximum m. gates row =
+// [input | forget] inputs (heads each); i = cap tanh((. + b) / cap), f = logsigmoid(cap tanh(.));
 // m' = max(f + m, i); coef row = [exp(f + m - m') | 0 | exp(i - m') | exp(-m')]; m lives in the item's slot.
+// A token is the map m -> max(m + f, i); two of them in a row are the map m -> max(m + (f1 + f2), max(i1 + f2, i2)),
+// so 64 tokens at a time are put together by a scan over the wave's lanes and applied to the m in front of them.
 __global__ __launch_bounds__(64) void matrix_memory_gates_kernel(const float* __restrict__ gates, const float* __restrict__ bias,
                                                                  float cap, float* __restrict__ coef, float* __restrict__ state,
                                                                  int64_t state_row, const int32_t* __restrict__ item_start,
                                                                  const int32_t* __restrict__ slots, int heads) {
-  const int item = blockIdx.x;
+  const int item = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int64_t s0 = item_start[item], s1 = item_start[item + 1];
-  for (int h = threadIdx.x; h < heads; h += blockDim.x) {
-    float* mp = state + static_cast<int64_t>(slots[item]) * state_row + h;
-    float m = *mp;
-    const float bi = bias[h], bf = bias[heads + h];
-    for (int64_t t = s0; t < s1; ++t) {
-      const float il = cap * tanhf((gates[t * 2 * heads + h] + bi) / cap);
-      const float fl = -softplus_f(-cap * tanhf((gates[t * 2 * heads + heads + h] + bf) / cap));
-      const float mn = fmaxf(fl + m, il);
+  float* mp = state + static_cast<int64_t>(slots[item]) * state_row + h;
+  float m = *mp;
+  const float bi = bias[h], bf = bias[heads + h];
+  for (int64_t t0 = s0; t0 < s1; t0 += kWave) {
+    const int64_t t = t0 + lane;
+    const bool valid = t < s1;
+    // A lane past the item's end is the map that changes nothing.
+    const float il = valid ? cap * tanhf((gates[t * 2 * heads + h] + bi) / cap) : -INFINITY;
+    const float fl = valid ? -softplus_f(-cap * tanhf((gates[t * 2 * heads + heads + h] + bf) / cap)) : 0.f;
+    float a = fl, b = il;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const float ap = __shfl_up(a, o, kWave), bp = __shfl_up(b, o, kWave);
+      if (lane >= o) {
+        b = fmaxf(bp + a, b);
+        a = ap + a;
+      }
+    }
+    const float mn = fmaxf(m + a, b);
+    float before = __shfl_up(mn, 1, kWave);
+    if (lane == 0) before = m;
+    if (valid) {
       float* c = coef + t * 4 * heads;
-      c[h] = expf(fl + m - mn);
+      c[h] = expf(fl + before - mn);
       c[heads + h] = 0.f;
       c[2 * heads + h] = expf(il - mn);
       c[3 * heads + h] = expf(-mn);
-      m = mn;
     }
-    *mp = m;
+    m = __shfl(mn, kWave - 1, kWave);
   }
+  if (lane == 0) *mp = m;
 }
 
 // grid (tokens), 256 threads: u row = [q * q_scale | k] (heads x dim each), vals row = per head [v | 1].
@@ -308,15 +319,18 @@ int psamd_hyper_read(void* stream, const float* streams, int count, const float*
   return check_launch("psamd_hyper_read");
 }
 
-int psamd_hyper_write(void* stream, float* streams, int count, const float* mix, const float* write, const void* delta,
-                      int delta_dtype, int slices, int64_t slice_stride, int64_t tokens, int hidden) {
-  PSAMD_REQUIRE(tokens >= 0 && hidden > 0 && count >= 1 && count <= kMaxStreams && slices >= 1, "bad sizes (at most 16 streams)");
-  PSAMD_REQUIRE(delta_dtype == kF32 || (delta_dtype == kBF16 && slices == 1), "the delta is one tensor or float slices");
+int psamd_hyper_write(void* stream, float* streams, int count, const float* mix, const float* write, const void* a,
+                      int a_dtype, int a_slices, int64_t a_stride, float a_scale, const void* b, int b_dtype, int b_slices,
+                      int64_t b_stride, float b_scale, int64_t tokens, int hidden) {
+  PSAMD_REQUIRE(tokens >= 0 && hidden > 0 && count >= 1 && count <= kMaxStreams && a_slices >= 1 && b_slices >= 1,
+                "bad sizes (at most 16 streams)");
+  PSAMD_REQUIRE((a_dtype == kF32 || (a_dtype == kBF16 && a_slices == 1)) && (b == nullptr || b_dtype == kF32 || (b_dtype == kBF16 && b_slices == 1)),
+                "an output is one tensor or float slices");
   const int64_t n = tokens * hidden;
   if (n == 0) return 0;
   PSAMD_REQUIRE(ceil_div(n, 256) <= 2147483647LL, "too large for one launch");
   hyper_write_kernel<<<dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-      streams, n, count, mix, write, delta, delta_dtype, slices, slice_stride, n);
+      streams, n, count, mix, write, a, a_dtype, a_slices, a_stride, a_scale, b, b_dtype, b_slices, b_stride, b_scale, n);
   return check_launch("psamd_hyper_write");
 }
 
@@ -370,7 +384,9 @@ int psamd_matrix_memory_gates(void* stream, const float* gates, const float* bia
                               int64_t state_row, const int32_t* item_start, const int32_t* slots, int items, int heads) {
   PSAMD_REQUIRE(items >= 0 && heads > 0 && cap > 0.f && state_row >= heads, "bad sizes");
   if (items == 0) return 0;
-  matrix_memory_gates_kernel<<<dim3(static_cast<unsigned>(items)), dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+  PSAMD_REQUIRE(heads <= 65535, "too many heads for one launch");
+  matrix_memory_gates_kernel<<<dim3(static_cast<unsigned>(items), static_cast<unsigned>(heads)), dim3(64), 0,
+                               static_cast<hipStream_t>(stream)>>>(
       gates, bias, cap, coef, state, state_row, item_start, slots, heads);
   return check_launch("psamd_matrix_memory_gates");
 }

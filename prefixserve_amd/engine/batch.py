@@ -94,6 +94,9 @@ class StepContext:
     # the run about to start belongs to.
     embedding_output: Any = None
     pass_index: int = 0
+    # Set by a block whose kernel adds a weighted sum of several outputs to the stream itself
+    # (``parts.base.WeightedDeltas``); a sub-layer made of several then hands them over one by one.
+    takes_weighted_deltas: bool = False
 
 
 class StepPacker:

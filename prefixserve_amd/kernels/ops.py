@@ -105,7 +105,7 @@ _SIGNATURES = {
     "psamd_short_conv_to": [_vp, _vp, _i32, _i64, _vp, _vp, _vp, _i32, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32],
     "psamd_stream_rms_norm": [_vp, _vp, _vp, _f32, _i64, _i32],
     "psamd_hyper_read": [_vp, _vp, _i32, _vp, _vp, _f32, _vp, _vp, _i32, _i64, _i32],
-    "psamd_hyper_write": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i64, _i64, _i32],
+    "psamd_hyper_write": [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i64, _f32, _vp, _i32, _i32, _i64, _f32, _i64, _i32],
     "psamd_weighted_sum": [_vp, _vp, _i32, _i32, _i64, _f32, _vp, _i32, _i32, _i64, _f32, _vp, _i64],
     "psamd_activation": [_vp, _vp, _i32, _i64, _i32],
     "psamd_gated_group_norm": [_vp, _vp, _vp, _i64, _vp, _i32, _vp, _i32, _i64, _vp, _i32, _f32, _vp, _i64, _i32],
@@ -846,15 +846,16 @@ class HipOps:
         self._ok(self.lib.psamd_hyper_read(self._stream(), streams.data_ptr(), count, read.data_ptr(), weight.data_ptr(), float(eps),
                                            _ptr(factor), out.data_ptr(), _code(out.dtype), t, h))
 
-    def hyper_write(self, streams, mix, write, delta) -> None:
-        """streams[t'] <- sum_s mix[s, t'] streams[s] + write[t'] delta, all copies at once from the old ones; delta is
-        [T, H] in a kernel dtype or [S, T, H] float32 slices."""
+    def hyper_write(self, streams, mix, write, delta, scale: float = 1.0, delta2=None, scale2: float = 0.0) -> None:
+        """streams[t'] <- sum_s mix[s, t'] streams[s] + write[t'] (scale delta + scale2 delta2), all copies at once from the
+        old ones; a delta is [T, H] in a kernel dtype or [S, T, H] float32 slices; delta2 may be None."""
         count, t, h = self._streams(streams, "hyper_write")
         self._need(mix.dtype == torch.float32 and tuple(mix.shape) == (count, count) and mix.is_contiguous()
                    and write.dtype == torch.float32 and write.numel() == count and write.is_contiguous(), "hyper_write: float32 parameters")
         dptr, dcode, slices, stride = self._delta_args(delta, t, h, delta.dtype)
+        d2 = (None, _F32, 1, 0) if delta2 is None else self._delta_args(delta2, t, h, delta2.dtype)
         self._ok(self.lib.psamd_hyper_write(self._stream(), streams.data_ptr(), count, mix.data_ptr(), write.data_ptr(), dptr, dcode,
-                                            max(slices, 1), stride, t, h))
+                                            max(slices, 1), stride, float(scale), d2[0], d2[1], max(d2[2], 1), d2[3], float(scale2), t, h))
 
     def weighted_sum(self, a, a_scale: float, b, b_scale: float, out) -> None:
         """out (float32 [T, H]) = a_scale * a + b_scale * b; a and b are [T, H] in a kernel dtype or [S, T, H] float32 slices."""

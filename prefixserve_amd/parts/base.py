@@ -120,6 +120,15 @@ class NormedRows:
 
 
 @dataclass
+class WeightedDeltas:
+    """What a sub-layer made of several hands to a block that says it takes such (``ctx.takes_weighted_deltas``): the
+    sum over ``parts`` of scale * delta, each delta in one of the forms ``Mixer.forward`` may return, to be formed
+    in 32-bit by the kernel that adds it to the stream. A block that does not say so gets the sum as one tensor."""
+
+    parts: "list[tuple[torch.Tensor, float]]"
+
+
+@dataclass
 class Runtime:
     """What every part needs to run: the device, the activation dtype (bfloat16 for
     serving, float32 for the exact path), the kernel bindings and the buffer store."""

@@ -7,7 +7,8 @@ from typing import TYPE_CHECKING, Any, Mapping
 
 import torch
 
-from .base import FeedForward, Mixer, Norm, Part, Runtime, StateNeed, Transform, WeightWant, register_block, register_transform
+from .base import (FeedForward, Mixer, Norm, Part, Runtime, StateNeed, Transform, WeightedDeltas, WeightWant, register_block,
+                   register_transform)
 
 if TYPE_CHECKING:
     from prefixserve_amd.engine.batch import StepContext
@@ -119,7 +120,14 @@ class HyperConnectionBlock:
             x = ws.get("block.x", (t, self.hidden_size), rt.dtype)
             ops.hyper_read(streams, con.read, norm.weight, norm.eps, x,
                            factor=self.conv_w[q].view(-1) if self.taps == 1 else None)
-        ops.hyper_write(streams, con.mix, con.write, run(x))
+        y = run(x)
+        if isinstance(y, WeightedDeltas):
+            if len(y.parts) == 2:
+                (a, sa), (b, sb) = y.parts
+                ops.hyper_write(streams, con.mix, con.write, a, sa, b, sb)
+                return
+            raise ValueError("the stream's kernel adds one output or the weighted sum of two")
+        ops.hyper_write(streams, con.mix, con.write, y)
 
     def forward(self, residual: torch.Tensor, pending: torch.Tensor | None, ctx: "StepContext", cache: Any,
                 state: torch.Tensor | None, writes_cache: bool) -> None:
@@ -130,6 +138,7 @@ class HyperConnectionBlock:
             raise ValueError(f"the block is made for {self.streams} streams, the model runs {streams.shape[0]}")
         ctx.stream_copy = None
         kept, ctx.residual = ctx.residual, None      # the sub-layers hand their output back: it goes into every copy
+        ctx.takes_weighted_deltas = True
         try:
             self._sublayer("mixer", 0, self.mixer_norm, streams, ctx, state,
                            lambda x: self.mixer.forward(x, ctx, cache, state, writes_cache))
@@ -138,6 +147,7 @@ class HyperConnectionBlock:
                                lambda x: self.feed_forward.forward(x, ctx))
         finally:
             ctx.residual = kept
+            ctx.takes_weighted_deltas = False
         return None
 
 

@@ -6,7 +6,7 @@ from typing import TYPE_CHECKING, Any, Mapping
 
 import torch
 
-from .base import CacheNeed, Mixer, PositionEncoding, Runtime, StateNeed, WeightWant, make, register_mixer
+from .base import CacheNeed, Mixer, PositionEncoding, Runtime, StateNeed, WeightedDeltas, WeightWant, make, register_mixer
 from .spec import PartSpec
 
 if TYPE_CHECKING:
@@ -81,7 +81,7 @@ class ParallelMixers(Mixer):
         return StateNeed((n,), torch.float32) if n else None
 
     def forward(self, x: torch.Tensor, ctx: "StepContext", cache: Any, state: torch.Tensor | None,
-                writes_cache: bool) -> torch.Tensor:
+                writes_cache: bool) -> "torch.Tensor | WeightedDeltas":
         rt = self.rt
         kept, ctx.residual = getattr(ctx, "residual", None), None       # both hand their output back: it is weighted first
         try:
@@ -89,6 +89,8 @@ class ParallelMixers(Mixer):
             b = self.right.forward(x, ctx, cache if self.cached is self.right else None, state, writes_cache)
         finally:
             ctx.residual = kept
+        if getattr(ctx, "takes_weighted_deltas", False):
+            return WeightedDeltas([(a, self.scales[0]), (b, self.scales[1])])       # the block's kernel forms the sum
         out = rt.workspace.get("parallel.delta", (1, x.shape[0], self.hidden_size), torch.float32)
         rt.ops.weighted_sum(a, self.scales[0], b, self.scales[1], out[0])
         return out

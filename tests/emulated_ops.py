@@ -338,8 +338,10 @@ class EmulatedOps:
         h = weight.float() * u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps)
         out.copy_((h if factor is None else h * factor).to(out.dtype))
 
-    def hyper_write(self, streams, mix, write, delta) -> None:
-        y = delta.float().sum(0) if delta.dim() == 3 else delta.float()
+    def hyper_write(self, streams, mix, write, delta, scale=1.0, delta2=None, scale2=0.0) -> None:
+        y = scale * (delta.float().sum(0) if delta.dim() == 3 else delta.float())
+        if delta2 is not None:
+            y = y + scale2 * (delta2.float().sum(0) if delta2.dim() == 3 else delta2.float())
         streams.copy_(torch.einsum("st,sxh->txh", mix, streams) + write[:, None, None] * y[None])
 
     def weighted_sum(self, a, a_scale, b, b_scale, out) -> None:

@@ -117,6 +117,10 @@ def test_streams_are_read_and_written(ops, dtype, s, t, h):
         PLAIN.hyper_write(want, mix, write, delta_rows)
         assert same(got, want)
     a, b = rnd(t, h, dtype=dtype, seed=10), rnd(2, t, h, seed=11)
+    got, want = streams.clone(), streams.clone()
+    ops.hyper_write(got, mix, write, a, 0.8, b, -1.5)                      # the weighted sum of two outputs
+    PLAIN.hyper_write(want, mix, write, a, 0.8, b, -1.5)
+    assert same(got, want)
     got, want = (torch.empty(t, h, device=DEV) for _ in range(2))
     ops.weighted_sum(a, 0.8, b, -1.5, got)
     PLAIN.weighted_sum(a, 0.8, b, -1.5, want)
@@ -251,7 +255,7 @@ def test_attention_with_kept_tokens_pooled_blocks_and_a_gate(ops, dtype, hq, hkv
             if block:
                 o.pool_kv_append(kv[0], pl, ctx, 0, 1, hkv, d, block)
             out = torch.empty(t, hq * d, dtype=dtype, device=DEV)
-            o.paged_attention(qkv, out, kv[0], ctx, 0, hq, hkv, d, 0.4, window, keep_first=keep,
+            o.paged_attention(qkv, out, kv[0], ctx, 0, hq, hkv, d, 0.4, window, keep_first=keep, exact_weights=k >= 2,
                               pooled=(pl, 1, block) if block else None, head_gate=gate if k % 2 == 0 else None)
             outs.append(out)
         assert same(outs[0], outs[1], dtype), (k, rel(outs[0].float().cpu(), outs[1].float().cpu()))
