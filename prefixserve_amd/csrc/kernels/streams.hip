@@ -34,33 +34,48 @@ __global__ __launch_bounds__(256) void stream_rms_norm_kernel(float* __restrict_
   for (int i = threadIdx.x; i < hidden; i += 256) row[i] = row[i] * inv * w[i];
 }
 
-// grid (tokens), 256 threads: u = sum_s read[s] streams[s, t, :]; out = u / rms(u) * w (* factor).
-template <typename O>
+// grid (tokens), 256 threads: u = sum_s read[s] streams[s, t, :]; out = u / rms(u) * w (* factor). u is formed
+// once and kept in LDS (hidden floats) between the sum of squares and the output. COUNT > 0: the number of streams
+// is known at compile time, so that a thread's loads of all streams are in flight together (a step of a few
+// tokens is a few workgroups, and what it costs is how many loads wait for one another); COUNT 0: any number.
+template <typename O, int COUNT>
 __global__ __launch_bounds__(256) void hyper_read_kernel(const float* __restrict__ streams, int64_t stream_stride, int count,
                                                          const float* __restrict__ read, const float* __restrict__ w, float eps,
                                                          const float* __restrict__ factor, O* __restrict__ out, int hidden) {
   __shared__ float scratch[4];
+  extern __shared__ float u_s[];
   const float* base = streams + static_cast<int64_t>(blockIdx.x) * hidden;
-  float a[kMaxStreams];
+  constexpr int N = COUNT > 0 ? COUNT : kMaxStreams;
+  const int n = COUNT > 0 ? COUNT : count;
+  float a[N];
 #pragma unroll
-  for (int s = 0; s < kMaxStreams; ++s) a[s] = s < count ? read[s] : 0.f;
+  for (int s = 0; s < N; ++s) a[s] = s < n ? read[s] : 0.f;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < hidden; i += 256) {
-    float u = 0.f;
+  for (int i0 = threadIdx.x; i0 < hidden; i0 += 1024) {
+    float u[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s)
-      if (s < count) u = fmaf(a[s], base[s * stream_stride + i], u);
-    ss = fmaf(u, u, ss);
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + 256 * j;
+      if (i < hidden) {
+#pragma unroll
+        for (int s = 0; s < N; ++s)
+          if (s < n) u[j] = fmaf(a[s], base[s * stream_stride + i], u[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = i0 + 256 * j;
+      if (i < hidden) {
+        u_s[i] = u[j];
+        ss = fmaf(u[j], u[j], ss);
+      }
+    }
   }
   ss = block_sum(ss, scratch, 4);
   const float inv = 1.f / sqrtf(ss / static_cast<float>(hidden) + eps);
   O* o = out + static_cast<int64_t>(blockIdx.x) * hidden;
-  for (int i = threadIdx.x; i < hidden; i += 256) {
-    float u = 0.f;
-#pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s)
-      if (s < count) u = fmaf(a[s], base[s * stream_stride + i], u);
-    float v = u * inv * w[i];
+  for (int i = threadIdx.x; i < hidden; i += 256) {       // a thread reads back what it wrote itself
+    float v = u_s[i] * inv * w[i];
     if (factor != nullptr) v *= factor[i];
     o[i] = from_float<O>(v);
   }
@@ -124,29 +139,33 @@ __global__ __launch_bounds__(256) void activation_kernel(A* __restrict__ x, int6
   x[e] = from_float<A>(v);
 }
 
-// One wave per (token, part): v = (y + skip[head] x) * silu(z); out = v / sqrt(mean(v^2) + eps) * weight.
-template <typename A>
+// v = (y + skip[head] x) * silu(z); out = v / sqrt(mean(v^2) + eps) * weight over each of `parts` equal parts of a row.
+// WAVES = 1: one wave per (token, part), four of them a workgroup; WAVES = 4: a whole workgroup per (token, part), for
+// parts of more than 256 entries (a row normalized as a whole by one wave is 64 rounds of loads in a row).
+template <typename A, int WAVES>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, const float* __restrict__ x,
                                                                int64_t x_row, const float* __restrict__ skip, int vdim,
                                                                const A* __restrict__ gate, int64_t gate_row,
                                                                const float* __restrict__ weight, int parts, int part, float eps,
                                                                A* __restrict__ out, int64_t pairs) {
-  const int lane = threadIdx.x & (kWave - 1);
-  const int64_t pair = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
-  if (pair >= pairs) return;
+  __shared__ float scratch[4];
+  constexpr int T = WAVES * kWave;
+  const int lane = threadIdx.x % T;
+  const int64_t pair = WAVES == 4 ? static_cast<int64_t>(blockIdx.x) : static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (pair >= pairs) return;                       // with WAVES = 4 the whole workgroup leaves together
   const int64_t t = pair / parts;
   const int c0 = static_cast<int>(pair - t * parts) * part;
   const int64_t inner = static_cast<int64_t>(parts) * part;
   float ss = 0.f;
-  for (int i = lane; i < part; i += kWave) {
+  for (int i = lane; i < part; i += T) {
     const int c = c0 + i;
     const float z = to_float<A>(gate[t * gate_row + c]);
     const float v = fmaf(skip[c / vdim], x[t * x_row + c], y[t * inner + c]) * z * sigmoid_f(z);
     ss = fmaf(v, v, ss);
   }
-  ss = wave_sum(ss);
+  ss = WAVES == 4 ? block_sum(ss, scratch, 4) : wave_sum(ss);
   const float inv = 1.f / sqrtf(ss / static_cast<float>(part) + eps);
-  for (int i = lane; i < part; i += kWave) {
+  for (int i = lane; i < part; i += T) {
     const int c = c0 + i;
     const float z = to_float<A>(gate[t * gate_row + c]);
     const float v = fmaf(skip[c / vdim], x[t * x_row + c], y[t * inner + c]) * z * sigmoid_f(z);
@@ -314,8 +333,20 @@ int psamd_hyper_read(void* stream, const float* streams, int count, const float*
   if (tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t stride = tokens * hidden;
-  PSAMD_BY_DTYPE(out_dtype, (hyper_read_kernel<A_><<<dim3(static_cast<unsigned>(tokens)), dim3(256), 0, s>>>(
-                                streams, stride, count, read, weight, eps, factor, static_cast<A_*>(out), hidden)));
+  const size_t smem = sizeof(float) * static_cast<size_t>(hidden);
+  PSAMD_REQUIRE(smem <= 60 * 1024, "rows of up to 15,360 numbers");
+#define PSAMD_READ(C_)                                                                                                   \
+  PSAMD_BY_DTYPE(out_dtype, (hyper_read_kernel<A_, C_><<<dim3(static_cast<unsigned>(tokens)), dim3(256), smem, s>>>(     \
+                                streams, stride, count, read, weight, eps, factor, static_cast<A_*>(out), hidden)))
+  switch (count) {
+    case 1: PSAMD_READ(1); break;
+    case 2: PSAMD_READ(2); break;
+    case 3: PSAMD_READ(3); break;
+    case 4: PSAMD_READ(4); break;
+    case 8: PSAMD_READ(8); break;
+    default: PSAMD_READ(0); break;
+  }
+#undef PSAMD_READ
   return check_launch("psamd_hyper_read");
 }
 
@@ -364,9 +395,16 @@ int psamd_gated_group_norm(void* stream, const float* y, const float* x, int64_t
   if (pairs == 0) return 0;
   PSAMD_REQUIRE(ceil_div(pairs, 4) <= 2147483647LL, "too large for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  PSAMD_BY_DTYPE(act_dtype, (gated_group_norm_kernel<A_><<<dim3(static_cast<unsigned>(ceil_div(pairs, 4))), dim3(256), 0, s>>>(
-                                y, x, x_row, skip, inner / heads, static_cast<const A_*>(gate), gate_row, weight, parts,
-                                inner / parts, eps, static_cast<A_*>(out), pairs)));
+  if (inner / parts > 256) {
+    PSAMD_REQUIRE(pairs <= 2147483647LL, "too large for one launch");
+    PSAMD_BY_DTYPE(act_dtype, (gated_group_norm_kernel<A_, 4><<<dim3(static_cast<unsigned>(pairs)), dim3(256), 0, s>>>(
+                                  y, x, x_row, skip, inner / heads, static_cast<const A_*>(gate), gate_row, weight, parts,
+                                  inner / parts, eps, static_cast<A_*>(out), pairs)));
+  } else {
+    PSAMD_BY_DTYPE(act_dtype, (gated_group_norm_kernel<A_, 1><<<dim3(static_cast<unsigned>(ceil_div(pairs, 4))), dim3(256), 0, s>>>(
+                                  y, x, x_row, skip, inner / heads, static_cast<const A_*>(gate), gate_row, weight, parts,
+                                  inner / parts, eps, static_cast<A_*>(out), pairs)));
+  }
   return check_launch("psamd_gated_group_norm");
 }
 
