@@ -178,6 +178,7 @@ int psamd_general_delta_prepare(void* stream, const void* rows, int act_dtype, i
 // S' = d S; S = S' + (ps p)(c^T S*) + k (xs x)^T, S* = S' if reads_decayed else S; out = S^T r. k, c, p, r: float
 // vectors of `dim` per (token, key group), rows key_row apart; dvec (or NULL) per (token, head), dscal / pscal /
 // xscal (or NULL = 1) per (token, head), rows scal_row apart; x [.., heads x vdim] rows x_row apart; out likewise.
+// reads_decayed 2 (with c = p = k and no dvec): the caller says that pscal is zero throughout, S = d S + k (xs x)^T.
 int psamd_delta_scan(void* stream, const float* kvec, const float* cvec, const float* pvec, const float* rvec, int64_t key_row,
                      int key_groups, const float* dvec, int64_t dvec_row, const float* dscal, const float* pscal,
                      const float* xscal, int64_t scal_row, const float* x, int64_t x_row, float* out, int64_t out_row,

@@ -222,8 +222,20 @@ __device__ __forceinline__ void scan_load(ScanToken<E, SAME>& t, const float* __
 }
 
 // One token: the column's E entries in s, the read-out returned (the same in all 16 lanes).
-template <int E, bool SAME, bool RD>
+template <int E, bool SAME, bool RD, bool NR>
 __device__ __forceinline__ float scan_step(const ScanToken<E, SAME>& t, float (&s)[E]) {
+  if constexpr (NR) {
+    // Nothing is taken out: S <- d S + k xw. The new column does not wait for a sum over the lanes;
+    // only the read-out (r . d S) + xw (r . k) does, and nothing waits for that.
+    float rd = 0.f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const float dec = t.ds * s[e];
+      rd = fmaf(t.r[e], dec, rd);
+      s[e] = fmaf(t.k[e], t.xw, dec);
+    }
+    return fmaf(t.xw, t.rk, row16_sum(rd));
+  }
   float dec[E];
   float dot = 0.f, rd = 0.f;
 #pragma unroll
@@ -254,17 +266,17 @@ __device__ __forceinline__ float scan_step(const ScanToken<E, SAME>& t, float (&
 
 // Tokens tk and tk + 1 of a run of n: the next token's operands are read from LDS while one is computed.
 // ta holds token tk on entry and token tk + 2 on exit.
-template <int E, bool SAME, bool RD>
+template <int E, bool SAME, bool RD, bool NR>
 __device__ __forceinline__ void scan_two(ScanToken<E, SAME>& ta, ScanToken<E, SAME>& tb, float (&s)[E], const float* __restrict__ vec,
                                          const float* __restrict__ sca, const float* __restrict__ xs, int tk, int n,
                                          float* __restrict__ o, int64_t out_row, int j, bool writes, int l, int col) {
   constexpr int TT = kScanRun<E>;
   scan_load(tb, vec, sca, xs, min(tk + 1, TT - 1), l, col);
-  const float ra = scan_step<E, SAME, RD>(ta, s);
+  const float ra = scan_step<E, SAME, RD, NR>(ta, s);
   if (writes) o[tk * out_row + j] = ra;
   if (tk + 1 < n) {
     scan_load(ta, vec, sca, xs, min(tk + 2, TT - 1), l, col);
-    const float rb = scan_step<E, SAME, RD>(tb, s);
+    const float rb = scan_step<E, SAME, RD, NR>(tb, s);
     if (writes) o[(tk + 1) * out_row + j] = rb;
   }
 }
@@ -277,7 +289,7 @@ __device__ __forceinline__ void scan_two(ScanToken<E, SAME>& ta, ScanToken<E, SA
 // take = ps (c . S*), the new column is dec + p take + k xw, and its read-out r . S is
 // (r . dec) + take (r . p) + xw (r . k), where r . dec is summed beside c . S* and the two
 // products of vectors alone are formed once per token for all columns when the run arrives.
-template <int E, bool SAME, bool RD>
+template <int E, bool SAME, bool RD, bool NR = false>
 __global__ __launch_bounds__(256) void delta_scan_kernel(
     const float* __restrict__ kvec, const float* __restrict__ cvec, const float* __restrict__ pvec,
     const float* __restrict__ rvec, int64_t key_row, int heads_per_group, const float* __restrict__ dvec, int64_t dvec_row,
@@ -375,9 +387,9 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
     scan_load(ta, vec, sca, xs_, 0, l, col);
     if (kScanUnrolled<E> && n == TT) {                  // a whole run: every LDS address and row offset is a constant
 #pragma unroll
-      for (int tk = 0; tk < TT; tk += 2) scan_two<E, SAME, RD>(ta, tb, s, vec, sca, xs_, tk, TT, o, out_row, j, writes, l, col);
+      for (int tk = 0; tk < TT; tk += 2) scan_two<E, SAME, RD, NR>(ta, tb, s, vec, sca, xs_, tk, TT, o, out_row, j, writes, l, col);
     } else {
-      for (int tk = 0; tk < n; tk += 2) scan_two<E, SAME, RD>(ta, tb, s, vec, sca, xs_, tk, n, o, out_row, j, writes, l, col);
+      for (int tk = 0; tk < n; tk += 2) scan_two<E, SAME, RD, NR>(ta, tb, s, vec, sca, xs_, tk, n, o, out_row, j, writes, l, col);
     }
   }
 #pragma unroll
@@ -413,13 +425,13 @@ __global__ __launch_bounds__(256) void heads_norm_gate_kernel(const float* __res
   }
 }
 
-template <int E, bool SAME, bool RD>
+template <int E, bool SAME, bool RD, bool NR = false>
 static int launch_delta_scan(hipStream_t s, dim3 grid, const float* kvec, const float* cvec, const float* pvec,
                              const float* rvec, int64_t key_row, int heads_per_group, const float* dvec, int64_t dvec_row,
                              const float* dscal, const float* pscal, const float* xscal, int64_t scal_row, const float* x,
                              int64_t x_row, float* out, int64_t out_row, float* state, int64_t state_row,
                              const int32_t* item_start, const int32_t* slots, int dim, int vdim) {
-  delta_scan_kernel<E, SAME, RD><<<grid, dim3(256), 0, s>>>(kvec, cvec, pvec, rvec, key_row, heads_per_group, dvec, dvec_row,
+  delta_scan_kernel<E, SAME, RD, NR><<<grid, dim3(256), 0, s>>>(kvec, cvec, pvec, rvec, key_row, heads_per_group, dvec, dvec_row,
                                                            dscal, pscal, xscal, scal_row, x, x_row, out, out_row, state,
                                                            state_row, item_start, slots, dim, vdim);
   return check_launch("psamd_delta_scan");
@@ -519,11 +531,14 @@ int psamd_delta_scan(void* stream, const float* kvec, const float* cvec, const f
   const int hpg = heads / key_groups;
   // The gated rule's form: one vector serves as key, direction and removal, the decay is a number per head.
   const bool same = cvec == kvec && pvec == kvec && dvec == nullptr && reads_decayed != 0;
+  // reads_decayed 2: nothing is taken out (the removal's scale is zero throughout), in the gated rule's form only.
+  PSAMD_REQUIRE(reads_decayed != 2 || same, "a recurrence without removal comes in the gated rule's form");
 #define PSAMD_SCAN_ARGS                                                                                                   \
   s, grid, kvec, cvec, pvec, rvec, key_row, hpg, dvec, dvec_row, dscal, pscal, xscal, scal_row, x, x_row, out, out_row, state, \
       state_row, item_start, slots, dim, vdim
 #define PSAMD_SCAN(E)                                                                                   \
-  return same ? launch_delta_scan<E, true, true>(PSAMD_SCAN_ARGS)                                       \
+  return same ? (reads_decayed == 2 ? launch_delta_scan<E, true, true, true>(PSAMD_SCAN_ARGS)           \
+                                    : launch_delta_scan<E, true, true>(PSAMD_SCAN_ARGS))                \
               : reads_decayed ? launch_delta_scan<E, false, true>(PSAMD_SCAN_ARGS)                      \
                               : launch_delta_scan<E, false, false>(PSAMD_SCAN_ARGS)
   switch (e) {

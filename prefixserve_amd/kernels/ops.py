@@ -988,7 +988,7 @@ class HipOps:
 
     def delta_scan(self, keys, directions, removals, queries, key_groups: int, decay_vectors, decay, removal_scale,
                    value_scale, values, out, state, state_offset: int, ctx, heads: int, dim: int, vdim: int,
-                   reads_decayed: bool) -> None:
+                   reads_decayed: bool, no_removal: bool = False) -> None:
         """The delta-rule recurrence over each item's tokens from its state slot. Every operand is a pair
         (float32 tensor [T, row], first column) or None. Per head h (its key group g = h // (heads / key_groups))
         and token: S' = d S with d = decay_vectors[h, :] (per key channel) times decay[h] (a number), either may
@@ -996,10 +996,15 @@ class HipOps:
         values[h])^T with S* = S' if ``reads_decayed`` else the S before the token; out[h] = S^T queries[g].
         ``keys``, ``directions``, ``removals``, ``queries`` lie in one tensor, as do ``decay``, ``removal_scale``,
         ``value_scale``. The state of head h is ``state[slot, state_offset + (h vdim + j) dim + i]``; out is
-        float32 [T, heads vdim]."""
+        float32 [T, heads vdim]. ``no_removal``: the caller says that ``removal_scale`` is zero throughout (a linear
+        recurrence S = d S + k (xs x)^T in the gated rule's form: keys, directions and removals one vector, a decay per
+        head); the kernel then skips the removal and the sum it waits for."""
         t = out.shape[0]
         self._need(t == ctx.num_tokens and out.dtype == torch.float32 and out.shape == (t, heads * vdim) and out.is_contiguous(),
                    "delta_scan: out is float32 [T, heads vdim]")
+        if no_removal:
+            self._need(reads_decayed and decay_vectors is None and keys[1] == directions[1] == removals[1],
+                       "delta_scan: without removal only in the gated rule's form")
         self._need(heads % key_groups == 0 and 1 <= dim <= 256 and vdim >= 1, "delta_scan: sizes")
         base = keys[0]
         for pair in (keys, directions, removals, queries):
@@ -1029,7 +1034,7 @@ class HipOps:
             at(decay_vectors), 0 if decay_vectors is None else decay_vectors[0].shape[1], at(decay), at(removal_scale),
             at(value_scale), 0 if sbase is None else sbase.shape[1], at(values), xv.shape[1], out.data_ptr(), out.shape[1],
             state.data_ptr() + 4 * state_offset, state.shape[1], ctx.item_start.data_ptr(), ctx.slots.data_ptr(),
-            ctx.num_items, heads, dim, vdim, int(reads_decayed)))
+            ctx.num_items, heads, dim, vdim, 2 if no_removal else int(reads_decayed)))
 
     def heads_norm_gate(self, o, heads: int, vdim: int, weight, weight_per_head: bool, eps: float, gate_rows, gate_col: int,
                         activation: str, out) -> None:

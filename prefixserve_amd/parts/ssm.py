@@ -96,7 +96,7 @@ class SelectiveStateSpace(Mixer):
         ops.delta_scan(keys=(u, b_col), directions=(u, b_col), removals=(u, b_col), queries=(u, b_col + self.groups * self.state_dim),
                        key_groups=self.groups, decay_vectors=None, decay=(coef, 0), removal_scale=(coef, hd),
                        value_scale=(coef, 2 * hd), values=(u, 0), out=y, state=state, state_offset=self.state_base + self.tail,
-                       ctx=ctx, heads=hd, dim=self.state_dim, vdim=self.value_dim, reads_decayed=True)
+                       ctx=ctx, heads=hd, dim=self.state_dim, vdim=self.value_dim, reads_decayed=True, no_removal=True)
         out = ws.get("ssm.out", (t, self.inner), rt.dtype)
         ops.gated_group_norm(y, u, 0, self.skip, hd, rows, 0, self.norm_w, self.norm_groups, self.norm_eps, out)
         return ops.linear_to_residual(out, self.w_o, "ssm.delta", getattr(ctx, "residual", None))
@@ -181,7 +181,7 @@ class MatrixMemory(Mixer):
         ops.delta_scan(keys=(u, k_col), directions=(u, k_col), removals=(u, k_col), queries=(u, 0), key_groups=hd,
                        decay_vectors=None, decay=(coef, 0), removal_scale=(coef, hd), value_scale=(coef, 2 * hd),
                        values=(vals, 0), out=raw, state=state, state_offset=self.state_base, ctx=ctx, heads=hd,
-                       dim=self.head_dim, vdim=vd, reads_decayed=True)
+                       dim=self.head_dim, vdim=vd, reads_decayed=True, no_removal=True)
         out = ws.get("memory.out", (t, self.value_size), rt.dtype)
         ops.memory_read_norm_gate(raw, coef, 3 * hd, hd, self.value_dim, self.READ_EPS, self.norm_w, self.norm_eps, rows,
                                   2 * self.key_size + self.value_size, out)

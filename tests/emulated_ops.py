@@ -289,7 +289,7 @@ class EmulatedOps:
         operands.copy_(torch.cat([r, k, v, w, -torch.sigmoid(a + rate_bias) * c, c], dim=-1))
 
     def delta_scan(self, keys, directions, removals, queries, key_groups, decay_vectors, decay, removal_scale,
-                   value_scale, values, out, state, state_offset, ctx, heads, dim, vdim, reads_decayed) -> None:
+                   value_scale, values, out, state, state_offset, ctx, heads, dim, vdim, reads_decayed, no_removal=False) -> None:
         t = out.shape[0]
 
         def vec(pair, n, size):

@@ -186,7 +186,7 @@ def test_state_space_layer_through_the_delta_scan(ops, dtype, heads, vdim, n, gr
             y = torch.empty(t, inner, device=DEV)
             o.delta_scan(keys=(u, inner), directions=(u, inner), removals=(u, inner), queries=(u, inner + groups * n),
                          key_groups=groups, decay_vectors=None, decay=(coef, 0), removal_scale=(coef, heads), value_scale=(coef, 2 * heads),
-                         values=(u, 0), out=y, state=state, state_offset=7, ctx=step, heads=heads, dim=n, vdim=vdim, reads_decayed=True)
+                         values=(u, 0), out=y, state=state, state_offset=7, ctx=step, heads=heads, dim=n, vdim=vdim, reads_decayed=True, no_removal=True)
             out = torch.empty(t, inner, dtype=dtype, device=DEV)
             o.gated_group_norm(y, u, 0, skip, heads, z, 3, norm_w, parts, 1e-5, out)
             outs.append((coef, y, out))
@@ -219,7 +219,7 @@ def test_matrix_memory_through_the_delta_scan(ops, dtype, heads, dim, vdim, cap)
             raw = torch.empty(t, heads * vd, device=DEV)
             o.delta_scan(keys=(u, ks), directions=(u, ks), removals=(u, ks), queries=(u, 0), key_groups=heads, decay_vectors=None,
                          decay=(coef, 0), removal_scale=(coef, heads), value_scale=(coef, 2 * heads), values=(vals, 0), out=raw,
-                         state=state, state_offset=4, ctx=step, heads=heads, dim=dim, vdim=vd, reads_decayed=True)
+                         state=state, state_offset=4, ctx=step, heads=heads, dim=dim, vdim=vd, reads_decayed=True, no_removal=True)
             out = torch.empty(t, vs, dtype=dtype, device=DEV)
             o.memory_read_norm_gate(raw, coef, 3 * heads, heads, vdim, 1e-6, norm_w, 1e-5, rows, 2 * ks + vs, out)
             outs.append((coef, u, vals, raw, out))
