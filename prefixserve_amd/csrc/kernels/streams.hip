@@ -126,17 +126,28 @@ __global__ __launch_bounds__(256) void weighted_sum_kernel(const void* __restric
 }
 
 // kind 0 = GELU (exact), 1 = GELU (tanh form), 2 = SiLU, 3 = ReLU.
+__device__ __forceinline__ float activate(float z, int kind) {
+  if (kind == 0) return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
+  if (kind == 1) return gelu_tanh_f(z);
+  if (kind == 2) return z * sigmoid_f(z);
+  return fmaxf(z, 0.f);
+}
+
+// Sixteen bytes per thread and access (8 bfloat16 or 4 floats); the entries behind the last whole group one by one.
 template <typename A>
 __global__ __launch_bounds__(256) void activation_kernel(A* __restrict__ x, int64_t n, int kind) {
-  const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (e >= n) return;
-  const float z = to_float<A>(x[e]);
-  float v;
-  if (kind == 0) v = 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
-  else if (kind == 1) v = gelu_tanh_f(z);
-  else if (kind == 2) v = z * sigmoid_f(z);
-  else v = fmaxf(z, 0.f);
-  x[e] = from_float<A>(v);
+  constexpr int V = 16 / sizeof(A);
+  const int64_t g = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t groups = n / V;
+  if (g < groups) {
+    uint4 raw = reinterpret_cast<uint4*>(x)[g];
+    A* v = reinterpret_cast<A*>(&raw);
+#pragma unroll
+    for (int i = 0; i < V; ++i) v[i] = from_float<A>(activate(to_float<A>(v[i]), kind));
+    reinterpret_cast<uint4*>(x)[g] = raw;
+  } else if (g == groups) {
+    for (int64_t e = groups * V; e < n; ++e) x[e] = from_float<A>(activate(to_float<A>(x[e]), kind));
+  }
 }
 
 // v = (y + skip[head] x) * silu(z); out = v / sqrt(mean(v^2) + eps) * weight over each of `parts` equal parts of a row.
@@ -299,7 +310,22 @@ __global__ __launch_bounds__(64) void pool_kv_append_kernel(const A* __restrict_
   const int off = slot % kPage;
   for (int i = threadIdx.x; i < d; i += kWave) {
     float ks = 0.f, vs = 0.f;
-    for (int j = pos - block + 1; j <= pos; ++j) {
+    int j = pos - block + 1;
+    for (; j + 3 <= pos; j += 4) {                       // four positions' loads in flight, added in the positions' order
+      float kq[4], vq[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const A* src = kv + static_cast<int64_t>(table[(j + q) / kPage]) * page_elems + static_cast<int64_t>(kvh) * kPage * d;
+        kq[q] = to_float<A>(src[((j + q) % kPage) * d + i]);
+        vq[q] = to_float<A>(src[half + static_cast<int64_t>(i) * kPage + ((j + q) % kPage)]);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        ks += kq[q];
+        vs += vq[q];
+      }
+    }
+    for (; j <= pos; ++j) {
       const A* src = kv + static_cast<int64_t>(table[j / kPage]) * page_elems + static_cast<int64_t>(kvh) * kPage * d;
       ks += to_float<A>(src[(j % kPage) * d + i]);
       vs += to_float<A>(src[half + static_cast<int64_t>(i) * kPage + (j % kPage)]);
@@ -382,7 +408,9 @@ int psamd_activation(void* stream, void* x, int act_dtype, int64_t n, int kind) 
   if (n == 0) return 0;
   PSAMD_REQUIRE(ceil_div(n, 256) <= 2147483647LL, "too large for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  PSAMD_BY_DTYPE(act_dtype, (activation_kernel<A_><<<dim3(static_cast<unsigned>(ceil_div(n, 256))), dim3(256), 0, s>>>(
+  PSAMD_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0, "the tensor must start at a multiple of 16 bytes");
+  const int64_t threads = n / (act_dtype == kBF16 ? 8 : 4) + 1;
+  PSAMD_BY_DTYPE(act_dtype, (activation_kernel<A_><<<dim3(static_cast<unsigned>(ceil_div(threads, 256))), dim3(256), 0, s>>>(
                                 static_cast<A_*>(x), n, kind)));
   return check_launch("psamd_activation");
 }
