@@ -145,9 +145,10 @@ class Engine:
         multiples of 8) by repeating its last item, when steps are replayed as graphs: a batch
         that loses one request at a time would otherwise meet a new shape, and a capture, at
         every step. The repeated item computes what the original computes and writes the same
-        values to the same place; its row of the result is not looked at."""
+        values to the same place; its row of the result is not looked at. Not with per-request state:
+        the repeated item would read the slot while the original replaces what is in it."""
         n = len(work)
-        if not self.runner.use_graphs or n == 0:
+        if not self.runner.use_graphs or n == 0 or self.runner.states:
             return work
         size = next((s for s in self._sizes if s >= n), n)
         return work + [work[-1]] * (size - n) if size > n else work
