@@ -238,7 +238,7 @@ int psamd_attention_masked(void* stream, const void* qkv, int q_stride, void* ou
                            const int32_t* block_ids, int hq, int hkv, int head_dim, float scale, int window, int keep_first,
                            const void* pool, const int32_t* pool_table_off, const int32_t* pool_block_ids, int block,
                            const float* gate);
-// The same on the matrix cores (bfloat16; shapes psamd_attention_mfma_supports takes): the step's portions as tiles
+// The same on the matrix cores (bfloat16; shapes psamd_attention_mfma_supports takes, head sizes up to 192): the step's portions as tiles
 // of 32 queries (pf_tiles) and its single tokens as tiles of one (dec_items).
 int psamd_attention_masked_mfma(void* stream, const void* qkv, int q_stride, void* out, const void* kv,
                                 const int32_t* pf_tiles, int n_tiles, const int32_t* dec_items, int n_dec, int max_kv_len,

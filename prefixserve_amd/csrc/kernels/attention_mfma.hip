@@ -1722,7 +1722,9 @@ int psamd_attention_masked_mfma(void* stream, const void* qkv, int q_stride, voi
     case 6: PSAMD_MASKED(6)
     case 7: PSAMD_MASKED(7)
     case 8: PSAMD_MASKED(8)
-    default: return fail("psamd_attention_masked_mfma: head sizes up to 128 (psamd_attention_masked takes the others)");
+    case 10: PSAMD_MASKED(10)
+    case 12: PSAMD_MASKED(12)
+    default: return fail("psamd_attention_masked_mfma: head sizes up to 192 (psamd_attention_masked takes the others)");
   }
 #undef PSAMD_MASKED
 #undef PSAMD_MASKED_LAUNCH

@@ -1105,7 +1105,7 @@ class HipOps:
             if head_gate is not None:
                 self._need(head_gate.dtype == torch.float32 and head_gate.shape == (t, hq) and head_gate.is_contiguous(),
                            "attention: the gate is float32 [T, hq]")
-            if (qkv.dtype == torch.bfloat16 and qkv.shape[1] % 8 == 0 and d <= 128 and self.mfma_attention_supported(hq, hkv, d)
+            if (qkv.dtype == torch.bfloat16 and qkv.shape[1] % 8 == 0 and d <= 192 and self.mfma_attention_supported(hq, hkv, d)
                     and self.MFMA_ATTENTION_EXTRAS and (self.fixed_kv_len or ctx.max_kv_len) <= 65536):
                 # The matrix cores: portions as tiles of 32 queries, single tokens as tiles of one.
                 kv_len = self.fixed_kv_len or ctx.max_kv_len

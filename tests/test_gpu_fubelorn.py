@@ -231,7 +231,7 @@ def test_matrix_memory_through_the_delta_scan(ops, dtype, heads, dim, vdim, cap)
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hq,hkv,d,window,keep,block", [(4, 2, 32, 9, 0, 4), (3, 3, 16, 6, 3, 0), (2, 1, 48, 70, 20, 16), (2, 2, 64, 3, 0, 7),
-                                                        (8, 2, 128, 40, 18, 1), (1, 1, 512, 5, 2, 3)])
+                                                        (8, 2, 128, 40, 18, 1), (2, 1, 160, 30, 3, 5), (4, 2, 192, 50, 8, 12), (1, 1, 512, 5, 2, 3)])
 def test_attention_with_kept_tokens_pooled_blocks_and_a_gate(ops, dtype, hq, hkv, d, window, keep, block):
     """Block means are written as their last token runs; then a portion, a single token and a new request see the window,
     the kept first tokens and the blocks wholly in front of the window, from pages in a scrambled order."""
