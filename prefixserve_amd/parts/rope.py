@@ -11,15 +11,15 @@ from .base import RotaryTable, Runtime, register_position
 
 
 def rope_inv_freq(head_dim: int, theta: float, scaling: Mapping[str, Any] | None) -> torch.Tensor:
+    """``rope_inv_freq64`` rounded once to float32, which agrees with the reference's float32
+    evaluation to one ulp and does not depend on a library's ``pow``."""
     return rope_inv_freq64(head_dim, theta, scaling).to(torch.float32)
 
 
 def rope_inv_freq64(head_dim: int, theta: float, scaling: Mapping[str, Any] | None) -> torch.Tensor:
     """inv_freq[i] = 1 / theta^(2i/D), i < D/2, then the llama3 three bands by wavelength:
     long waves divided by ``factor``, short ones unchanged, the middle blended
-    (prefixserve/model/llama.py:24-46 of the reference). Evaluated in float64 and rounded
-    once to float32, which agrees with the reference's float32 evaluation to one ulp and
-    does not depend on a library's ``pow``."""
+    (prefixserve/model/llama.py:24-46 of the reference). Evaluated and returned in float64."""
     i = torch.arange(0, head_dim, 2, dtype=torch.float64)
     inv = 1.0 / (torch.tensor(float(theta), dtype=torch.float64) ** (i / head_dim))
     if scaling is not None:
